@@ -377,6 +377,220 @@ def mekevik_preset(name: str, width: int, vocab: int, pattern: str,
                          logit_scale=logit_scale)
 
 
+# ---------------------------------------------------------------------------
+# Feditar: a per-layer decoder of RECURRENT mixers on an fp32 residual
+# stream.  The embedding adds a hashed (previous, current) token-pair row
+# and a learned position row; every layer is pre-norm (RMS, weight stored
+# around zero) around one mixer and an optional relu^2 feed-forward.
+# Mixers: an mLSTM matrix memory, a Mamba-2 state-space layer, or a
+# PARALLEL pair — causal softmax attention (short convolutions on q/k/v,
+# position-dependent query stretch, tanh score cap) beside an RWKV-style
+# decayed outer-product memory — whose normed outputs are averaged.
+# ---------------------------------------------------------------------------
+@dataclass
+class PairHashSpec:
+    """Row of the pair table for (previous, current):
+    (prev * mul_prev + cur * mul_cur) mod buckets; a sequence's first
+    token takes row `buckets` (the table has buckets + 1 rows)."""
+    buckets: int = 1
+    mul_prev: int = 1
+    mul_cur: int = 1
+
+
+@dataclass
+class MLSTMSpec:
+    heads: int = 1
+    dim: int = 64              # query/key entries per head
+    vdim: int = 64             # value entries per head
+    gate_cap: float = 15.0     # gates pass through cap * tanh(. / cap)
+
+
+@dataclass
+class Mamba2Spec:
+    heads: int = 1
+    vdim: int = 64             # channels per head (inner = heads * vdim)
+    state: int = 64            # state entries per channel
+    groups: int = 1            # B / C groups shared by heads
+    conv: int = 4              # taps of the short convolution
+    norm_groups: int = 1       # equal parts of the gated output norm
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+@dataclass
+class SoftcapAttentionSpec:
+    heads: int = 1
+    kv_heads: int = 1
+    dim: int = 64
+    vdim: int = 64
+    scale: float = 0.0         # 0 => dim ** -0.5
+    softcap: float = 0.0       # 0 => scores are not squashed
+    conv: int = 1              # taps of the q/k/v convolutions; 1 = none
+    temp_coef: float = 0.0     # query *= 1 + coef * ln(floor((p+1)/every)+1)
+    temp_every: int = 1
+
+    def __post_init__(self):
+        if not self.scale:
+            self.scale = float(self.dim) ** -0.5
+
+
+@dataclass
+class DecayMemorySpec:
+    """RWKV-style time mixing: per-channel decays from a low-rank map."""
+    heads: int = 1
+    dim: int = 64              # key = value entries per head
+    decay_rank: int = 16
+
+
+@dataclass
+class ParallelMixerSpec:
+    left: SoftcapAttentionSpec = None
+    right: DecayMemorySpec = None
+
+
+@dataclass
+class Relu2FFSpec:
+    ff: int = 0
+
+
+@dataclass
+class FeditarConfig:
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: list               # LayerSpec(type="mlstm"|"mamba2"|"parallel")
+    norm_eps: float = 1e-6
+    embed_scale: float = 1.0
+    pair_hash: PairHashSpec = None
+    max_position: int = 2048   # rows of the learned position table
+    architecture: str = "Feditar"
+
+    def __post_init__(self):
+        if self.pair_hash is None:
+            self.pair_hash = PairHashSpec()
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return False
+
+    def kv_bytes_per_token(self, itemsize: int = 2) -> int:
+        """Paged bytes per token: only the attention half of a parallel
+        mixer pages anything; everything else is fixed per slot."""
+        return max(itemsize, sum(
+            l.mixer.left.kv_heads * (l.mixer.left.dim + l.mixer.left.vdim)
+            * itemsize for l in self.layers if l.type == "parallel"))
+
+    @staticmethod
+    def from_dict(cfg: dict, name: str = "feditar",
+                  shapes: Optional[dict] = None) -> "FeditarConfig":
+        """Parse the design's config.json.  `shapes` (tensor name ->
+        shape, from the checkpoint header) gives what the json leaves
+        to the tensors (rank of the decay map)."""
+        shapes = shapes or {}
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m = l.get("mixer") or {}
+            t = l["type"]
+            if t == "mlstm":
+                mixer = MLSTMSpec(heads=int(m["heads"]), dim=int(m["dim"]),
+                                  vdim=int(m.get("vdim") or m["dim"]),
+                                  gate_cap=float(m["gate_cap"]))
+            elif t == "mamba2":
+                mixer = Mamba2Spec(
+                    heads=int(m["heads"]), vdim=int(m["vdim"]),
+                    state=int(m["state"]), groups=int(m.get("groups") or 1),
+                    conv=int(m["conv"]),
+                    norm_groups=int(m.get("norm_groups") or 1))
+            elif t == "parallel":
+                a, b = m["left"], m["right"]
+                qt = a.get("q_temp") or {}
+                w1 = shapes.get(f"l{i}.mix.right.w1")
+                mixer = ParallelMixerSpec(
+                    left=SoftcapAttentionSpec(
+                        heads=int(a["heads"]),
+                        kv_heads=int(a.get("kv_heads") or a["heads"]),
+                        dim=int(a["dim"]),
+                        vdim=int(a.get("vdim") or a["dim"]),
+                        scale=float(a.get("scale") or 0.0),
+                        softcap=float(a.get("softcap") or 0.0),
+                        conv=int(a.get("conv") or 1),
+                        temp_coef=float(qt.get("coef") or 0.0),
+                        temp_every=int(qt.get("every") or 1)),
+                    right=DecayMemorySpec(
+                        heads=int(b["heads"]), dim=int(b["dim"]),
+                        decay_rank=int(w1[0]) if w1 else int(
+                            b.get("decay_rank", 16))))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer {t!r}")
+            f = l.get("mlp")
+            if f is None:
+                mlp = None
+            elif f["kind"] == "dense":
+                mlp = Relu2FFSpec(ff=int(f["ff"]))
+            else:
+                raise ValueError(f"layer {i}: unknown mlp {f['kind']!r}")
+            layers.append(LayerSpec(type=t, mixer=mixer, mlp=mlp))
+        e = cfg.get("embedding") or {}
+        bg = e.get("bigram") or {}
+        return FeditarConfig(
+            name=name, hidden_size=int(cfg["width"]),
+            vocab_size=int(cfg["vocab"]), layers=layers,
+            norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-6)),
+            embed_scale=float(e.get("scale", 1.0)),
+            pair_hash=PairHashSpec(buckets=int(bg.get("buckets", 1)),
+                                   mul_prev=int(bg.get("mul_prev", 1)),
+                                   mul_cur=int(bg.get("mul_cur", 1))),
+            max_position=int(cfg.get("max_positions", 2048)))
+
+
+def feditar_preset(name: str, width: int, vocab: int, pattern: str,
+                   heads: int, dim: int, vdim: int, kv_heads: int = 0,
+                   state: int = 64, groups: int = 1, ff: int = 0,
+                   conv: int = 4, norm_groups: int = 1,
+                   decay_rank: int = 32, gate_cap: float = 15.0,
+                   softcap: float = 50.0, temp_coef: float = 0.1,
+                   temp_every: int = 128, buckets: int = 4093,
+                   max_position: int = 4096) -> FeditarConfig:
+    """Layer pattern string: one letter pair per layer — mixer `x`
+    (mLSTM), `s` (Mamba-2) or `p` (parallel attention + decayed
+    memory), then feed-forward `d` (relu^2) or `-` (none); e.g.
+    "x- s- pd"."""
+    layers = []
+    for tok in pattern.split():
+        if tok[0] == "x":
+            typ, mixer = "mlstm", MLSTMSpec(heads=heads, dim=dim, vdim=vdim,
+                                            gate_cap=gate_cap)
+        elif tok[0] == "s":
+            typ, mixer = "mamba2", Mamba2Spec(
+                heads=heads, vdim=vdim, state=state, groups=groups,
+                conv=conv, norm_groups=norm_groups)
+        else:
+            typ, mixer = "parallel", ParallelMixerSpec(
+                left=SoftcapAttentionSpec(
+                    heads=heads, kv_heads=kv_heads or heads, dim=dim,
+                    vdim=vdim, softcap=softcap, conv=conv,
+                    temp_coef=temp_coef, temp_every=temp_every),
+                right=DecayMemorySpec(heads=heads, dim=dim,
+                                      decay_rank=decay_rank))
+        mlp = Relu2FFSpec(ff=ff) if tok[1] == "d" else None
+        layers.append(LayerSpec(type=typ, mixer=mixer, mlp=mlp))
+    return FeditarConfig(
+        name=name, hidden_size=width, vocab_size=vocab, layers=layers,
+        embed_scale=float(width) ** 0.5,
+        pair_hash=PairHashSpec(buckets=buckets, mul_prev=8191, mul_cur=131),
+        max_position=max_position)
+
+
 # Architectures from the public model cards (random-init weights — no network).
 MODEL_PRESETS = {
     "llama-3-8b": ModelConfig(
@@ -525,6 +739,16 @@ MODEL_PRESETS = {
         "mekevik-4k", width=4096, vocab=32000, pattern="d m d m",
         heads=32, kv_heads=8, dim=128, vdim=128, window=4096, ff=14336,
         experts=8, top=2, expert_ff=14336, bias_rows=64, bias_far=4096.0),
+    "tiny-feditar": feditar_preset(
+        "tiny-feditar", width=96, vocab=320, pattern="x- s- pd s-",
+        heads=4, kv_heads=2, dim=16, vdim=24, state=8, groups=2, ff=160,
+        conv=3, norm_groups=2, decay_rank=8, gate_cap=8.0, softcap=20.0,
+        temp_coef=0.25, temp_every=8, buckets=211, max_position=512),
+    # layer-shape benchmark point at Llama-3-8B's width
+    "feditar-4k": feditar_preset(
+        "feditar-4k", width=4096, vocab=32000, pattern="x- s- pd pd",
+        heads=32, kv_heads=8, dim=128, vdim=128, state=128, groups=8,
+        ff=14336, norm_groups=8, decay_rank=64),
     "tiny-moe": ModelConfig(
         name="tiny-moe",
         hidden_size=512,
@@ -652,6 +876,19 @@ class EngineConfig:
     def tiny_mekevik(**kw) -> "EngineConfig":
         defaults = dict(
             model=MODEL_PRESETS["tiny-mekevik"],
+            num_gpu_blocks=64,
+            max_num_seqs=8,
+            max_batched_tokens=2048,
+            max_model_len=512,
+            use_hip_graphs=False,
+        )
+        defaults.update(kw)
+        return EngineConfig(**defaults)
+
+    @staticmethod
+    def tiny_feditar(**kw) -> "EngineConfig":
+        defaults = dict(
+            model=MODEL_PRESETS["tiny-feditar"],
             num_gpu_blocks=64,
             max_num_seqs=8,
             max_batched_tokens=2048,

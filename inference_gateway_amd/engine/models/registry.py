@@ -8,7 +8,8 @@ from pathlib import Path
 
 import torch
 
-from ..config import FedatarConfig, MekevikConfig, ModelConfig
+from ..config import (FedatarConfig, FeditarConfig, MekevikConfig,
+                      ModelConfig)
 
 
 def build_model(model_cfg, device, dtype):
@@ -17,6 +18,8 @@ def build_model(model_cfg, device, dtype):
         from .fedatar import FedatarForCausalLM as cls
     elif isinstance(model_cfg, MekevikConfig):
         from .mekevik import MekevikForCausalLM as cls
+    elif isinstance(model_cfg, FeditarConfig):
+        from .feditar import FeditarForCausalLM as cls
     elif model_cfg.is_moe:
         from .mixtral import MixtralForCausalLM as cls
     else:
@@ -53,6 +56,10 @@ def model_config_from_dir(path: str):
         return MekevikConfig.from_dict(
             cfg, name=Path(path).name or "mekevik",
             shapes=safetensors_shapes(path))
+    if cfg.get("architecture") == "Feditar":
+        return FeditarConfig.from_dict(
+            cfg, name=Path(path).name or "feditar",
+            shapes=safetensors_shapes(path))
     if cfg.get("architecture") == "Fedatar":
         return FedatarConfig.from_dict(
             cfg, name=Path(path).name or "fedatar",
@@ -66,9 +73,12 @@ def is_recurrent(model_cfg) -> bool:
     """True when some layer keeps per-sequence state outside the paged
     cache (prefix reuse across requests is then impossible: the state at
     a shared prefix's end is not stored)."""
+    if isinstance(model_cfg, FeditarConfig):
+        return True     # every mixer and the embedding keep slot state
     return isinstance(model_cfg, FedatarConfig) and any(
         l.type == "mingru" for l in model_cfg.layers)
 
 
 __all__ = ["build_model", "model_config_from_dir", "safetensors_shapes",
-           "is_recurrent", "ModelConfig", "FedatarConfig", "MekevikConfig"]
+           "is_recurrent", "ModelConfig", "FedatarConfig", "MekevikConfig",
+           "FeditarConfig"]

@@ -396,6 +396,93 @@ def load_mekevik_weights(model, path: str) -> int:
     return n
 
 
+def load_feditar_weights(model, path: str) -> int:
+    """Load a Feditar checkpoint: tensors `embed`, `bigram`, `pos`,
+    `embed.norm`, `l<i>.norm1|norm2`, `l<i>.mix.*` per mixer kind,
+    `l<i>.mlp.{up,down}`, `final.norm`.  The engine's layouts are
+    assembled here: q|k|v|g stacked for the matrix memory's input GEMM
+    and its two gate rows (with biases) kept apart in fp32; the
+    state-space input projection split into its z|x|B|C rows and its
+    fp32 step-size rows; q|k|v and their convolution filters stacked for
+    the attention half of a parallel mixer; the decayed memory's four
+    projections stacked K-major.  Norm weights stored around zero are
+    held as 1 + w."""
+    sh = _Shards(path)
+    cfg = model.cfg
+    n = 0
+
+    def put(param, src, what):
+        nonlocal n
+        _copy(param, src, what)
+        n += 1
+
+    def one_plus(name):
+        return 1.0 + sh.full(name).float()
+
+    put(model.embed, sh.full("embed"), "embed")
+    put(model.pair, sh.full("bigram"), "bigram")
+    put(model.pos, sh.full("pos"), "pos")
+    put(model.embed_norm_w, one_plus("embed.norm"), "embed.norm")
+    for i, (spec, layer) in enumerate(zip(cfg.layers, model.layers)):
+        p = f"l{i}."
+        put(layer.norm1_w, one_plus(p + "norm1"), p + "norm1")
+        mx, m = layer.mixer, p + "mix."
+        if spec.type == "mlstm":
+            put(mx.qkvg, torch.cat([sh.full(m + c) for c in "qkvg"], 0),
+                m + "q|k|v|g")
+            put(mx.gates_w, torch.cat([sh.full(m + "i"), sh.full(m + "f")],
+                                      0), m + "i|f")
+            put(mx.gates_b, torch.cat([sh.full(m + "i.b"),
+                                       sh.full(m + "f.b")], 0), m + "i|f.b")
+            put(mx.norm_w, sh.full(m + "norm"), m + "norm")
+            put(mx.o, sh.full(m + "o"), m + "o")
+        elif spec.type == "mamba2":
+            rows = spec.mixer.inner + spec.mixer.conv_channels
+            w_in = sh.full(m + "in")
+            if w_in.shape[0] != rows + spec.mixer.heads:
+                raise ValueError(
+                    f"{m}in: checkpoint has {w_in.shape[0]} rows, the "
+                    f"configuration needs {rows + spec.mixer.heads}")
+            put(mx.in_main, w_in[:rows], m + "in[z|x|B|C]")
+            put(mx.dt_w, w_in[rows:], m + "in[dt]")
+            put(mx.dt_b, sh.full(m + "dt_bias"), m + "dt_bias")
+            put(mx.conv_w, sh.full(m + "conv"), m + "conv")
+            put(mx.conv_b, sh.full(m + "conv.b"), m + "conv.b")
+            put(mx.a_log, sh.full(m + "A_log"), m + "A_log")
+            put(mx.skip, sh.full(m + "D"), m + "D")
+            put(mx.norm_w, sh.full(m + "norm"), m + "norm")
+            put(mx.o, sh.full(m + "o"), m + "o")
+        elif spec.type == "parallel":
+            a, ml = mx.left, m + "left."
+            put(a.qkv, torch.cat([sh.full(ml + c) for c in "qkv"], 0),
+                ml + "q|k|v")
+            if spec.mixer.left.conv > 1:
+                put(a.conv_w, torch.cat(
+                    [sh.full(ml + c + ".conv") for c in "qkv"], 0),
+                    ml + "q|k|v.conv")
+            put(a.o, sh.full(ml + "o"), ml + "o")
+            b, mr = mx.right, m + "right."
+            put(b.mu, torch.stack([sh.full(mr + "mu." + c)
+                                   for c in b.MIXES]), mr + "mu.*")
+            put(b.rkvg_t, torch.stack([sh.full(mr + c).t() for c in "rkvg"]),
+                mr + "r|k|v|g")
+            put(b.w1, sh.full(mr + "w1"), mr + "w1")
+            put(b.w2, sh.full(mr + "w2"), mr + "w2")
+            put(b.w0, sh.full(mr + "w0"), mr + "w0")
+            put(b.bonus, sh.full(mr + "u"), mr + "u")
+            put(b.norm_w, sh.full(mr + "norm"), mr + "norm")
+            put(b.o, sh.full(mr + "o"), mr + "o")
+            put(mx.left_out, sh.full(ml + "out"), ml + "out")
+            put(mx.right_out, sh.full(mr + "out"), mr + "out")
+        if spec.mlp is None:
+            continue
+        put(layer.norm2_w, one_plus(p + "norm2"), p + "norm2")
+        put(layer.mlp.up, sh.full(p + "mlp.up"), p + "mlp.up")
+        put(layer.mlp.down, sh.full(p + "mlp.down"), p + "mlp.down")
+    put(model.final_norm_w, one_plus("final.norm"), "final.norm")
+    return n
+
+
 def _is_gguf(path: str) -> bool:
     p = Path(path)
     if p.is_file():
@@ -419,6 +506,8 @@ def load_weights(model, path: str) -> int:
         return load_fedatar_weights(model, path)
     if getattr(model.cfg, "architecture", "") == "Mekevik":
         return load_mekevik_weights(model, path)
+    if getattr(model.cfg, "architecture", "") == "Feditar":
+        return load_feditar_weights(model, path)
     if getattr(model.cfg, "is_moe", False):
         return load_mixtral_weights(model, path)
     return load_llama_weights(model, path)

@@ -31,6 +31,35 @@ except ImportError:  # pragma: no cover - absent only before first build
     HAS_HYBRID = False
 
 
+try:
+    from . import _recurrent  # matrix-memory / state-space / decay mixers
+
+    HAS_RECURRENT = True
+except ImportError:  # pragma: no cover - absent only before first build
+    _recurrent = None
+    HAS_RECURRENT = False
+
+
+def _require_recurrent() -> None:
+    if not HAS_RECURRENT:
+        raise RuntimeError(
+            "inference_gateway_amd.ops._recurrent is not built but a GPU "
+            "tensor was passed. Build it in-tree with: "
+            "IGW_BUILD_EXT=recurrent PYTORCH_ROCM_ARCH=gfx950 python "
+            "setup.py build_ext --inplace"
+        )
+
+
+def _shared_ext(name: str):
+    """The row-wise ops that both the hybrid and the recurrent extension
+    compile (same source file): whichever is loaded serves them, so a
+    process that runs one model family loads one library."""
+    for ext in (_hybrid, _recurrent):
+        if ext is not None and hasattr(ext, name):
+            return getattr(ext, name)
+    _require_hybrid()
+
+
 def _require_hybrid() -> None:
     if not HAS_HYBRID:
         raise RuntimeError(
@@ -419,9 +448,8 @@ def xielu(z, pq):
 
 def relu2(z):
     if z.is_cuda:
-        _require_hybrid()
         out = torch.empty_like(z)
-        _hybrid.relu2(out, z)
+        _shared_ext("relu2")(out, z)
         return out
     return torch_ref.relu2_ref(z)
 
@@ -478,12 +506,11 @@ def add_rmsnorm_pair(residual, delta_a, delta_b, w1, w2, eps: float,
     be None).  Returns (rmsnorm(residual) * w1, rmsnorm(residual) * w2)
     from ONE pass and one statistic; w2 None gives (out, None)."""
     if residual.is_cuda:
-        _require_hybrid()
         out1 = torch.empty(residual.shape, dtype=out_dtype,
                            device=residual.device)
         out2 = None if w2 is None else torch.empty_like(out1)
-        _hybrid.add_rmsnorm_pair(out1, out2, residual, delta_a, delta_b,
-                                 w1, w2, eps)
+        _shared_ext("add_rmsnorm_pair")(out1, out2, residual, delta_a,
+                                        delta_b, w1, w2, eps)
         return out1, out2
     return torch_ref.add_rmsnorm_pair_ref(residual, delta_a, delta_b, w1,
                                           w2, eps, out_dtype)
@@ -570,3 +597,210 @@ def gated_act(gate_up, mode: int, limit: float = 0.0, alpha: float = 1.0):
         _hybrid.gated_act(out, gate_up, mode, limit, alpha)
         return out
     return torch_ref.gated_act_ref(gate_up, mode, limit, alpha)
+
+
+# ---------------------------------------------------------------------------
+# Recurrent mixers (extension _recurrent, CPU versions in recurrent_ref):
+# matrix memories, state-space layers, decayed outer-product memories,
+# short convolutions, and softmax attention with a score cap.  Every op
+# takes the ragged-batch description of ForwardBatch (seq_cu, seq_start,
+# seq_slots) and keeps per-sequence state in slot buffers; a sequence
+# whose first row is position 0 starts from zero.
+# ---------------------------------------------------------------------------
+from . import recurrent_ref  # noqa: E402
+
+DECAY_LINEAR = recurrent_ref.DECAY_LINEAR
+DECAY_EXP_NEG_EXP = recurrent_ref.DECAY_EXP_NEG_EXP
+GATE_SIGMOID = recurrent_ref.GATE_SIGMOID
+GATE_SILU = recurrent_ref.GATE_SILU
+
+
+def embed_pair_norm(token_ids, positions, prev_tok, seq_cu, seq_start,
+                    seq_slots, row_seq, embed, pair, pos, norm_w,
+                    scale: float, buckets: int, mul_prev: int, mul_cur: int,
+                    eps: float):
+    """fp32 residual [T, D] = rmsnorm(embed[tok] * scale + pair[hash(prev,
+    tok)] + pos[position]) * norm_w.  hash = (prev * mul_prev + tok *
+    mul_cur) mod buckets; a sequence's first token reads row `buckets`.
+    prev_tok [slots, 1] int32 carries each sequence's last token."""
+    if embed.is_cuda:
+        _require_recurrent()
+        out = torch.empty((token_ids.shape[0], embed.shape[1]),
+                          dtype=torch.float32, device=embed.device)
+        _recurrent.embed_pair_norm(out, token_ids, positions, prev_tok,
+                                   seq_cu, seq_start, seq_slots, row_seq,
+                                   embed, pair, pos, norm_w, scale, buckets,
+                                   mul_prev, mul_cur, eps)
+        return out
+    return recurrent_ref.embed_pair_norm_ref(
+        token_ids, positions, prev_tok, seq_cu, seq_start, seq_slots, embed,
+        pair, pos, norm_w, scale, buckets, mul_prev, mul_cur, eps)
+
+
+def causal_conv(x, w, bias, state, seq_cu, seq_start, seq_slots, row_seq,
+                silu: bool):
+    """Per-channel causal filter over each sequence's rows: x [T, C]
+    (strided rows ok), w [C, taps] fp32 (last tap = current row), bias
+    [C] fp32 or None, optional silu.  state [slots, (taps-1)*C] fp32
+    holds every sequence's last taps-1 inputs."""
+    if x.is_cuda:
+        _require_recurrent()
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _recurrent.causal_conv(out, x, w, bias, state, seq_cu, seq_start,
+                               seq_slots, row_seq, silu)
+        return out
+    return recurrent_ref.causal_conv_ref(x, w, bias, state, seq_cu,
+                                         seq_start, seq_slots, silu)
+
+
+def token_shift_mix(h, mu, state, seq_cu, seq_start, seq_slots, row_seq):
+    """[S, T, D]: h + (h_prev - h) * mu[s] for each of the S mixing
+    vectors; h_prev = previous row of the sequence (state [slots, D] fp32
+    across steps, zeros at position 0)."""
+    if h.is_cuda:
+        _require_recurrent()
+        out = torch.empty((mu.shape[0],) + tuple(h.shape), dtype=h.dtype,
+                          device=h.device)
+        _recurrent.token_shift_mix(out, h, mu, state, seq_cu, seq_start,
+                                   seq_slots, row_seq)
+        return out
+    return recurrent_ref.token_shift_mix_ref(h, mu, state, seq_cu,
+                                             seq_start, seq_slots)
+
+
+def mlstm_gates(pre, cap: float, m_state, seq_cu, seq_start, seq_slots):
+    """Stabilised exponential gates of a matrix memory from fp32
+    pre-activations [T, 2H] (input | forget); m_state [slots, H] fp32 is
+    the running maximum.  Returns fp32 (decay, kscale, floor) [T, H]."""
+    if pre.is_cuda:
+        _require_recurrent()
+        T, H = pre.shape[0], pre.shape[1] // 2
+        out = torch.empty((3, T, H), dtype=torch.float32, device=pre.device)
+        _recurrent.mlstm_gates(out, pre, cap, m_state, seq_cu, seq_start,
+                               seq_slots)
+        return out[0], out[1], out[2]
+    return recurrent_ref.mlstm_gates_ref(pre, cap, m_state, seq_cu,
+                                         seq_start, seq_slots)
+
+
+def ssm_gates(dt_pre, a_log):
+    """Step sizes and decays of a state-space layer from fp32
+    pre-activations [T, H] (bias included): dt = softplus(dt_pre), decay =
+    exp(-exp(a_log) * dt).  Returns fp32 (decay, dt)."""
+    if dt_pre.is_cuda:
+        _require_recurrent()
+        out = torch.empty((2,) + tuple(dt_pre.shape), dtype=torch.float32,
+                          device=dt_pre.device)
+        _recurrent.ssm_gates(out, dt_pre, a_log)
+        return out[0], out[1]
+    dt = torch.nn.functional.softplus(dt_pre, threshold=40.0)
+    return torch.exp(-torch.exp(a_log) * dt), dt
+
+
+def outer_scan(q, k, v, decay, kscale, bonus, skip, state, seq_cu,
+               seq_start, seq_slots, seq_rows, decay_mode: int = 0,
+               ones_col: bool = False, qscale: float = 1.0):
+    """Outer-product memory per (sequence, head), S [N, PP] fp32 in
+    state [slots, H*N*PP]:  S' = diag(a_t) S + (kscale_t k_t) v_t^T;
+    o_t = S'^T q_t, or with `bonus` u [H, N] the look-before-write form
+    o_t = (S + diag(u) k_t v_t^T)^T q_t; o_t = o_t * qscale + skip_h v_t.
+    q, k [T, G, N] (strided ok; head h reads group h // (H/G)), v [T, H,
+    P], decay fp32 [T, H, 1 | N] holding a_t (DECAY_LINEAR) or x with a_t
+    = exp(-exp(x)) (DECAY_EXP_NEG_EXP); ones_col appends a column of ones
+    to v (PP = P + 1: the memory's normaliser).  Returns fp32 [T, H, PP].
+    seq_rows: python row counts (host side, picks the launch shape)."""
+    if v.is_cuda:
+        _require_recurrent()
+        T, H, P = v.shape
+        out = torch.empty((T, H, P + (1 if ones_col else 0)),
+                          dtype=torch.float32, device=v.device)
+        _recurrent.outer_scan(out, q, k, v, decay, kscale, bonus, skip,
+                              state, seq_cu, seq_start, seq_slots,
+                              decay_mode, ones_col, qscale)
+        return out
+    return recurrent_ref.outer_scan_ref(
+        q, k, v, decay, kscale, bonus, skip, state, seq_cu, seq_start,
+        seq_slots, decay_mode, ones_col, qscale)
+
+
+def head_norm_gate(o, gate, w, eps: float, group: int, gate_act: int,
+                   gate_first: bool, floor, out_dtype):
+    """Epilogue of a memory read-out o fp32 [T, H, PP]: optional division
+    by max(|last column|, floor) + 1e-6 (floor [T, H] fp32), RMS norm in
+    groups of `group` channels times w [C] fp32, and a sigmoid or silu
+    gate from pre-activations gate [T, C] (strided ok) applied before or
+    after the norm.  Returns [T, C] in out_dtype."""
+    if o.is_cuda:
+        _require_recurrent()
+        T, H, PP = o.shape
+        C = H * (PP - (1 if floor is not None else 0))
+        out = torch.empty((T, C), dtype=out_dtype, device=o.device)
+        _recurrent.head_norm_gate(out, o, gate, w, eps, group, gate_act,
+                                  gate_first, floor)
+        return out
+    return recurrent_ref.head_norm_gate_ref(o, gate, w, eps, group, gate_act,
+                                            gate_first, floor, out_dtype)
+
+
+def append_paged_kv(k, v, kcache, vcache, slot_mapping):
+    """k [T, G*N], v [T, G*P] (strided rows ok) into paged caches
+    [blocks, G, block, N] and [blocks, G, block, P]."""
+    if k.is_cuda:
+        _require_recurrent()
+        _recurrent.append_paged_kv(k, v, kcache, vcache, slot_mapping)
+        return
+    recurrent_ref.append_paged_kv_ref(k, v, kcache, vcache, slot_mapping)
+
+
+# bf16 batches run the MFMA tile kernel when the sizes fit; off = the
+# wave-per-(row, head) kernel for everything
+SOFTCAP_ATTENTION_MFMA = True
+
+
+def softcap_attention(q, kcache, vcache, block_table, row_seq, positions,
+                      scale: float, softcap: float = 0.0,
+                      temp_coef: float = 0.0, temp_every: int = 1,
+                      window: int = 0, num_prefill_rows: int = 0,
+                      prefill_seq_lens=None, max_context: int = 0):
+    """Causal softmax attention over paged keys/values with grouped
+    heads and separate key and value widths.  score = (q . k) * scale *
+    (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)), squashed by
+    softcap * tanh(. / softcap) when softcap > 0; window > 0 keeps the
+    last `window` keys.  q [T, H*N] (strided ok) -> [T, H*P]."""
+    if q.is_cuda:
+        _require_recurrent()
+        T = q.shape[0]
+        H = q.shape[1] // kcache.shape[3]
+        out = torch.empty((T, H * vcache.shape[3]), dtype=q.dtype,
+                          device=q.device)
+        if (q.dtype == torch.bfloat16 and SOFTCAP_ATTENTION_MFMA
+                and hasattr(_recurrent, "softcap_attention_mfma")):
+            tq = _recurrent.softcap_attention_tile_rows()
+            tiles = _attention_tiles(
+                tq, num_prefill_rows,
+                tuple(prefill_seq_lens or ()) if num_prefill_rows else (),
+                T, q.device)
+            if _recurrent.softcap_attention_mfma(
+                    out, q, kcache, vcache, block_table, row_seq, positions,
+                    tiles[0], tiles[1], scale, softcap, temp_coef,
+                    temp_every, window, max_context or 4096,
+                    num_prefill_rows):
+                return out
+        _recurrent.softcap_attention(out, q, kcache, vcache, block_table,
+                                     row_seq, positions, scale, softcap,
+                                     temp_coef, temp_every, window)
+        return out
+    return recurrent_ref.softcap_attention_ref(
+        q, kcache, vcache, block_table, row_seq, positions, scale, softcap,
+        temp_coef, temp_every, window)
+
+
+def rmsnorm_pair_mean(a, b, wa, wb, eps: float):
+    """0.5 * (rmsnorm(a) * wa + rmsnorm(b) * wb): the two branches of a
+    parallel mixer, each normed over the model width, averaged."""
+    if a.is_cuda:
+        _require_recurrent()
+        out = torch.empty_like(a)
+        _recurrent.rmsnorm_pair_mean(out, a, b, wa, wb, eps)
+        return out
+    return recurrent_ref.rmsnorm_pair_mean_ref(a, b, wa, wb, eps)

@@ -1,0 +1,581 @@
+// Row-wise kernels of the recurrent mixers (gfx950).
+//
+//   embed_pair_norm    token row * scale + hashed (previous, current) pair
+//                      row + position row, RMS norm -> fp32 residual
+//   causal_conv        short per-channel causal filter over ragged
+//                      sequences, history in a slot buffer
+//   token_shift_mix    h + (h_prev - h) * mu for several mixing vectors
+//   mlstm_gates        capped exponential gates with a running maximum
+//   ssm_gates          softplus step sizes and their decays
+//   head_norm_gate     read-out epilogue: normaliser division, grouped
+//                      RMS norm, sigmoid / silu gate
+//   append_paged_kv    keys and values of unequal width into pages
+//   rmsnorm_pair_mean  average of two RMS-normed branches
+//
+// A batch is ragged: rows of sequence s are [seq_cu[s], seq_cu[s+1]), its
+// first row sits at position seq_start[s], its state in row seq_slots[s]
+// of a slot buffer.  A sequence that starts at position 0 reads no state.
+// All arithmetic is fp32; loads and stores are in the activation type.
+#include "../csrc_hybrid/act_types.h"
+
+namespace igw {
+
+constexpr int RROW_BLOCK = 256;
+
+DEVINLINE float rrow_block_sum(float x, float* lds) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  x = wave_reduce_sum(x);
+  __syncthreads();  // lds may still be read from a previous reduction
+  if (lane == 0) lds[wave] = x;
+  __syncthreads();
+  float r = 0.0f;
+#pragma unroll
+  for (int w = 0; w < RROW_BLOCK / 64; ++w) r += lds[w];
+  return r;
+}
+
+DEVINLINE float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
+// ---------------------------------------------------------------------------
+// embedding
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(RROW_BLOCK) void embed_pair_norm_kernel(
+    float* __restrict__ out, const int64_t* __restrict__ tokens,
+    const int32_t* __restrict__ positions, int32_t* __restrict__ prev_tok,
+    const int32_t* __restrict__ seq_cu, const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
+    const T* __restrict__ embed, const T* __restrict__ pair,
+    const T* __restrict__ pos, const float* __restrict__ w, int D,
+    int pos_rows, float scale, int64_t buckets, int64_t mul_prev,
+    int64_t mul_cur, float eps) {
+  __shared__ float lds[RROW_BLOCK / 64];
+  const int t = blockIdx.x;
+  const int s = row_seq[t];
+  const int r0 = seq_cu[s], r1 = seq_cu[s + 1];
+  const int64_t tok = tokens[t];
+  int64_t prow;
+  if (t > r0) {
+    prow = (tokens[t - 1] * mul_prev + tok * mul_cur) % buckets;
+  } else {
+    // the sequence's first row of this step: the only reader of the slot,
+    // and its writer (the step's last token)
+    const int slot = seq_slots[s];
+    if (seq_start[s] > 0)
+      prow = ((int64_t)prev_tok[slot] * mul_prev + tok * mul_cur) % buckets;
+    else
+      prow = buckets;
+    __syncthreads();
+    if (threadIdx.x == 0) prev_tok[slot] = (int32_t)tokens[r1 - 1];
+  }
+  const int p = min(positions[t], pos_rows - 1);
+  const T* e = embed + tok * D;
+  const T* b = pair + prow * D;
+  const T* q = pos + (int64_t)p * D;
+  float* o = out + (int64_t)t * D;
+  float sq = 0.0f;
+  for (int d = threadIdx.x; d < D; d += RROW_BLOCK) {
+    const float x = Act<T>::ld(e + d) * scale + Act<T>::ld(b + d) +
+                    Act<T>::ld(q + d);
+    o[d] = x;
+    sq += x * x;
+  }
+  const float rstd = 1.0f / sqrtf(rrow_block_sum(sq, lds) / (float)D + eps);
+  for (int d = threadIdx.x; d < D; d += RROW_BLOCK) o[d] = o[d] * rstd * w[d];
+}
+
+void embed_pair_norm(torch::Tensor out, torch::Tensor tokens,
+                     torch::Tensor positions, torch::Tensor prev_tok,
+                     torch::Tensor seq_cu, torch::Tensor seq_start,
+                     torch::Tensor seq_slots, torch::Tensor row_seq,
+                     torch::Tensor embed, torch::Tensor pair, torch::Tensor pos,
+                     torch::Tensor w, double scale, int64_t buckets,
+                     int64_t mul_prev, int64_t mul_cur, double eps) {
+  const int T = tokens.numel(), D = embed.size(1);
+  TORCH_CHECK(out.is_cuda() && out.dtype() == torch::kFloat32 &&
+              out.is_contiguous() && out.size(0) == T && out.size(1) == D);
+  TORCH_CHECK(tokens.dtype() == torch::kInt64 && tokens.is_contiguous());
+  TORCH_CHECK(positions.dtype() == torch::kInt32 && positions.numel() == T);
+  TORCH_CHECK(prev_tok.dtype() == torch::kInt32 && prev_tok.is_contiguous());
+  TORCH_CHECK(row_seq.dtype() == torch::kInt32 && row_seq.numel() == T);
+  TORCH_CHECK(seq_cu.dtype() == torch::kInt32 &&
+              seq_start.dtype() == torch::kInt32 &&
+              seq_slots.dtype() == torch::kInt32);
+  TORCH_CHECK(embed.is_contiguous() && pair.is_contiguous() &&
+              pos.is_contiguous() && pair.size(1) == D && pos.size(1) == D &&
+              pair.dtype() == embed.dtype() && pos.dtype() == embed.dtype());
+  TORCH_CHECK(pair.size(0) == buckets + 1, "pair table needs buckets+1 rows");
+  TORCH_CHECK(w.dtype() == torch::kFloat32 && w.numel() == D);
+  if (T == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  IGW_DISPATCH_ACT(embed, {
+    hipLaunchKernelGGL(
+        (embed_pair_norm_kernel<act_t>), dim3(T), dim3(RROW_BLOCK), 0, stream,
+        (float*)out.data_ptr(), (const int64_t*)tokens.data_ptr(),
+        (const int32_t*)positions.data_ptr(), (int32_t*)prev_tok.data_ptr(),
+        (const int32_t*)seq_cu.data_ptr(), (const int32_t*)seq_start.data_ptr(),
+        (const int32_t*)seq_slots.data_ptr(),
+        (const int32_t*)row_seq.data_ptr(), (const act_t*)embed.data_ptr(),
+        (const act_t*)pair.data_ptr(), (const act_t*)pos.data_ptr(),
+        (const float*)w.data_ptr(), D, (int)pos.size(0), (float)scale, buckets,
+        mul_prev, mul_cur, (float)eps);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------------------------------
+// short causal convolution
+// ---------------------------------------------------------------------------
+constexpr int CONV_MAX_TAPS = 8;
+
+// one thread per (row, channel): y = sum_j w[c, j] * u[t - taps + 1 + j]
+// with u = this step's rows, the slot history before them, zeros before
+// the sequence's start
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(
+    T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
+    const float* __restrict__ w, const float* __restrict__ bias,
+    const float* __restrict__ state, const int32_t* __restrict__ seq_cu,
+    const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
+    int C, int taps, int silu) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int s = row_seq[t];
+  const int r0 = seq_cu[s];
+  const bool has_hist = seq_start[s] > 0;
+  const float* hist = state + (int64_t)seq_slots[s] * (taps - 1) * C;
+  float acc = bias ? bias[c] : 0.0f;
+  for (int j = 0; j < taps; ++j) {
+    const int r = t - taps + 1 + j;
+    float u = 0.0f;
+    if (r >= r0) {
+      u = Act<T>::ld(x + (int64_t)r * x_stride + c);
+    } else if (has_hist) {
+      // history row index: taps-1 rows, oldest first; row r0-1 is the last
+      u = hist[(int64_t)(taps - 1 - (r0 - r)) * C + c];
+    }
+    acc += w[c * taps + j] * u;
+  }
+  if (silu) acc = silu_f32(acc);
+  Act<T>::st(out + (int64_t)t * C + c, acc);
+}
+
+// one thread per (sequence, channel): history <- last taps-1 inputs
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(
+    const T* __restrict__ x, int64_t x_stride, float* __restrict__ state,
+    const int32_t* __restrict__ seq_cu, const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, int C, int taps) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int r0 = seq_cu[s], r1 = seq_cu[s + 1];
+  const int n = r1 - r0;
+  if (n == 0) return;
+  float* hist = state + (int64_t)seq_slots[s] * (taps - 1) * C;
+  const bool has_hist = seq_start[s] > 0;
+  float old[CONV_MAX_TAPS];
+#pragma unroll
+  for (int j = 0; j < CONV_MAX_TAPS; ++j)
+    old[j] = (j < taps - 1 && has_hist) ? hist[(int64_t)j * C + c] : 0.0f;
+#pragma unroll
+  for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+    if (j >= taps - 1) break;
+    // new history row j is input index n - (taps-1) + j of this step
+    const int i = n - (taps - 1) + j;
+    float v;
+    if (i >= 0) {
+      v = Act<T>::ld(x + (int64_t)(r0 + i) * x_stride + c);
+    } else {
+      const int k = j + n;  // old row j + n (shifted by the new rows)
+      v = 0.0f;
+#pragma unroll
+      for (int m = 0; m < CONV_MAX_TAPS; ++m)
+        if (m == k) v = old[m];
+    }
+    hist[(int64_t)j * C + c] = v;
+  }
+}
+
+void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                 c10::optional<torch::Tensor> bias, torch::Tensor state,
+                 torch::Tensor seq_cu, torch::Tensor seq_start,
+                 torch::Tensor seq_slots, torch::Tensor row_seq, bool silu) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.stride(1) == 1);
+  const int T = x.size(0), C = x.size(1), taps = w.size(1);
+  const int S = seq_slots.numel();
+  TORCH_CHECK(out.is_contiguous() && out.dtype() == x.dtype() &&
+              out.size(0) == T && out.size(1) == C);
+  TORCH_CHECK(w.dtype() == torch::kFloat32 && w.is_contiguous() &&
+              w.size(0) == C);
+  TORCH_CHECK(taps >= 1 && taps <= CONV_MAX_TAPS + 1, "taps out of range");
+  if (bias.has_value())
+    TORCH_CHECK(bias->dtype() == torch::kFloat32 && bias->numel() == C);
+  TORCH_CHECK(state.dtype() == torch::kFloat32 && state.is_contiguous() &&
+              state.size(1) >= (int64_t)(taps - 1) * C);
+  TORCH_CHECK(state.size(1) == (int64_t)(taps - 1) * C || taps == 1,
+              "history buffer width must be (taps-1)*channels");
+  TORCH_CHECK(row_seq.dtype() == torch::kInt32 && row_seq.numel() == T);
+  TORCH_CHECK(seq_cu.dtype() == torch::kInt32 && seq_cu.numel() == S + 1 &&
+              seq_start.dtype() == torch::kInt32 && seq_start.numel() == S &&
+              seq_slots.dtype() == torch::kInt32);
+  if (T == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  IGW_DISPATCH_ACT(x, {
+    hipLaunchKernelGGL(
+        (causal_conv_kernel<act_t>), dim3((C + 255) / 256, T), dim3(256), 0,
+        stream, (act_t*)out.data_ptr(), (const act_t*)x.data_ptr(),
+        (int64_t)x.stride(0), (const float*)w.data_ptr(),
+        bias.has_value() ? (const float*)bias->data_ptr() : nullptr,
+        (const float*)state.data_ptr(), (const int32_t*)seq_cu.data_ptr(),
+        (const int32_t*)seq_start.data_ptr(),
+        (const int32_t*)seq_slots.data_ptr(),
+        (const int32_t*)row_seq.data_ptr(), C, taps, silu ? 1 : 0);
+    if (taps > 1)
+      hipLaunchKernelGGL(
+          (conv_state_kernel<act_t>), dim3((C + 255) / 256, S), dim3(256), 0,
+          stream, (const act_t*)x.data_ptr(), (int64_t)x.stride(0),
+          (float*)state.data_ptr(), (const int32_t*)seq_cu.data_ptr(),
+          (const int32_t*)seq_start.data_ptr(),
+          (const int32_t*)seq_slots.data_ptr(), C, taps);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------------------------------
+// token shift
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_mix_kernel(
+    T* __restrict__ out, const T* __restrict__ h, const float* __restrict__ mu,
+    float* __restrict__ state, const int32_t* __restrict__ seq_cu,
+    const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
+    int Trows, int D, int M) {
+  const int t = blockIdx.y;
+  const int d = blockIdx.x * 256 + threadIdx.x;
+  if (d >= D) return;
+  const int s = row_seq[t];
+  const int r0 = seq_cu[s];
+  const float cur = Act<T>::ld(h + (int64_t)t * D + d);
+  float prev;
+  if (t > r0) {
+    prev = Act<T>::ld(h + (int64_t)(t - 1) * D + d);
+  } else {
+    // first row of the sequence in this step: sole reader and writer of
+    // the slot entry
+    float* st = state + (int64_t)seq_slots[s] * D + d;
+    prev = seq_start[s] > 0 ? *st : 0.0f;
+    *st = Act<T>::ld(h + (int64_t)(seq_cu[s + 1] - 1) * D + d);
+  }
+  const float diff = prev - cur;
+  for (int m = 0; m < M; ++m)
+    Act<T>::st(out + ((int64_t)m * Trows + t) * D + d,
+               cur + diff * mu[m * D + d]);
+}
+
+void token_shift_mix(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
+                     torch::Tensor state, torch::Tensor seq_cu,
+                     torch::Tensor seq_start, torch::Tensor seq_slots,
+                     torch::Tensor row_seq) {
+  TORCH_CHECK(h.is_cuda() && h.is_contiguous() && h.dim() == 2);
+  const int T = h.size(0), D = h.size(1), M = mu.size(0);
+  TORCH_CHECK(out.is_contiguous() && out.dtype() == h.dtype() &&
+              out.numel() == (int64_t)M * T * D);
+  TORCH_CHECK(mu.dtype() == torch::kFloat32 && mu.is_contiguous() &&
+              mu.size(1) == D);
+  TORCH_CHECK(state.dtype() == torch::kFloat32 && state.is_contiguous() &&
+              state.size(1) == D);
+  TORCH_CHECK(row_seq.dtype() == torch::kInt32 && row_seq.numel() == T);
+  TORCH_CHECK(seq_cu.dtype() == torch::kInt32 &&
+              seq_start.dtype() == torch::kInt32 &&
+              seq_slots.dtype() == torch::kInt32);
+  if (T == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  IGW_DISPATCH_ACT(h, {
+    hipLaunchKernelGGL(
+        (token_shift_mix_kernel<act_t>), dim3((D + 255) / 256, T), dim3(256),
+        0, stream, (act_t*)out.data_ptr(), (const act_t*)h.data_ptr(),
+        (const float*)mu.data_ptr(), (float*)state.data_ptr(),
+        (const int32_t*)seq_cu.data_ptr(), (const int32_t*)seq_start.data_ptr(),
+        (const int32_t*)seq_slots.data_ptr(),
+        (const int32_t*)row_seq.data_ptr(), T, D, M);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------------------------------
+// gates
+// ---------------------------------------------------------------------------
+DEVINLINE float logsigmoid_f32(float x) {
+  // -softplus(-x), stable on both sides
+  return fminf(x, 0.0f) - log1pf(expf(-fabsf(x)));
+}
+
+// one thread per (sequence, head), rows in order
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(
+    float* __restrict__ out, const float* __restrict__ pre,
+    float* __restrict__ m_state, const int32_t* __restrict__ seq_cu,
+    const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, int T, int H, int S, float cap) {
+  const int idx = blockIdx.x * 64 + threadIdx.x;
+  if (idx >= S * H) return;
+  const int s = idx / H, h = idx % H;
+  const int r0 = seq_cu[s], r1 = seq_cu[s + 1];
+  if (r1 == r0) return;
+  float* ms = m_state + (int64_t)seq_slots[s] * H + h;
+  float m = seq_start[s] > 0 ? *ms : 0.0f;
+  const float inv_cap = 1.0f / cap;
+  float* decay = out;
+  float* kscale = out + (int64_t)T * H;
+  float* floor_ = out + (int64_t)2 * T * H;
+  for (int t = r0; t < r1; ++t) {
+    const float gi = cap * tanhf(pre[(int64_t)t * 2 * H + h] * inv_cap);
+    const float gf =
+        logsigmoid_f32(cap * tanhf(pre[(int64_t)t * 2 * H + H + h] * inv_cap));
+    const float m_new = fmaxf(gf + m, gi);
+    decay[(int64_t)t * H + h] = expf(gf + m - m_new);
+    kscale[(int64_t)t * H + h] = expf(gi - m_new);
+    floor_[(int64_t)t * H + h] = expf(-m_new);
+    m = m_new;
+  }
+  *ms = m;
+}
+
+void mlstm_gates(torch::Tensor out, torch::Tensor pre, double cap,
+                 torch::Tensor m_state, torch::Tensor seq_cu,
+                 torch::Tensor seq_start, torch::Tensor seq_slots) {
+  TORCH_CHECK(pre.is_cuda() && pre.dtype() == torch::kFloat32 &&
+              pre.is_contiguous() && pre.dim() == 2 && pre.size(1) % 2 == 0);
+  const int T = pre.size(0), H = pre.size(1) / 2, S = seq_slots.numel();
+  TORCH_CHECK(out.dtype() == torch::kFloat32 && out.is_contiguous() &&
+              out.numel() == (int64_t)3 * T * H);
+  TORCH_CHECK(m_state.dtype() == torch::kFloat32 && m_state.is_contiguous() &&
+              m_state.size(1) == H);
+  TORCH_CHECK(seq_cu.dtype() == torch::kInt32 && seq_cu.numel() == S + 1 &&
+              seq_start.dtype() == torch::kInt32 &&
+              seq_slots.dtype() == torch::kInt32);
+  if (T == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3((S * H + 63) / 64), dim3(64), 0,
+                     stream, (float*)out.data_ptr(),
+                     (const float*)pre.data_ptr(), (float*)m_state.data_ptr(),
+                     (const int32_t*)seq_cu.data_ptr(),
+                     (const int32_t*)seq_start.data_ptr(),
+                     (const int32_t*)seq_slots.data_ptr(), T, H, S, (float)cap);
+  HIP_CHECK_KERNEL();
+}
+
+__global__ __launch_bounds__(256) void ssm_gates_kernel(
+    float* __restrict__ out, const float* __restrict__ dt_pre,
+    const float* __restrict__ a_log, int64_t n, int H) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float x = dt_pre[i];
+  // softplus, stable on both sides
+  const float dt = fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x)));
+  out[i] = expf(-expf(a_log[i % H]) * dt);
+  out[n + i] = dt;
+}
+
+void ssm_gates(torch::Tensor out, torch::Tensor dt_pre, torch::Tensor a_log) {
+  TORCH_CHECK(dt_pre.is_cuda() && dt_pre.dtype() == torch::kFloat32 &&
+              dt_pre.is_contiguous() && dt_pre.dim() == 2);
+  const int64_t n = dt_pre.numel();
+  const int H = dt_pre.size(1);
+  TORCH_CHECK(out.dtype() == torch::kFloat32 && out.is_contiguous() &&
+              out.numel() == 2 * n);
+  TORCH_CHECK(a_log.dtype() == torch::kFloat32 && a_log.numel() == H);
+  if (n == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  hipLaunchKernelGGL(ssm_gates_kernel, dim3((n + 255) / 256), dim3(256), 0,
+                     stream, (float*)out.data_ptr(),
+                     (const float*)dt_pre.data_ptr(),
+                     (const float*)a_log.data_ptr(), n, H);
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------------------------------
+// read-out epilogue: one wave per (row, norm group)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(
+    T* __restrict__ out, const float* __restrict__ o,
+    const T* __restrict__ gate, int64_t gate_stride,
+    const float* __restrict__ w, const float* __restrict__ floor_, int H,
+    int P, int PP, int group, float eps, int gate_silu, int gate_first) {
+  const int t = blockIdx.y, g = blockIdx.x, lane = threadIdx.x;
+  const int C = H * P;
+  const int c0 = g * group;
+  const float* orow = o + (int64_t)t * H * PP;
+  const T* grow = gate + (int64_t)t * gate_stride;
+  float sq = 0.0f;
+  // pass 1: the value before the norm, and its square sum
+  for (int i = lane; i < group; i += 64) {
+    const int c = c0 + i;
+    const int h = c / P, p = c % P;
+    float v = orow[h * PP + p];
+    if (floor_ != nullptr) {
+      const float den =
+          fmaxf(fabsf(orow[h * PP + P]), floor_[(int64_t)t * H + h]) + 1e-6f;
+      v = v / den;
+    }
+    if (gate_first) {
+      const float z = Act<T>::ld(grow + c);
+      v *= gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
+    }
+    sq += v * v;
+  }
+  const float rstd = 1.0f / sqrtf(wave_reduce_sum(sq) / (float)group + eps);
+  for (int i = lane; i < group; i += 64) {
+    const int c = c0 + i;
+    const int h = c / P, p = c % P;
+    float v = orow[h * PP + p];
+    if (floor_ != nullptr) {
+      const float den =
+          fmaxf(fabsf(orow[h * PP + P]), floor_[(int64_t)t * H + h]) + 1e-6f;
+      v = v / den;
+    }
+    const float z = Act<T>::ld(grow + c);
+    const float gz = gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
+    if (gate_first) v *= gz;
+    v = v * rstd * w[c];
+    if (!gate_first) v *= gz;
+    Act<T>::st(out + (int64_t)t * C + c, v);
+  }
+}
+
+void head_norm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
+                    torch::Tensor w, double eps, int64_t group,
+                    int64_t gate_act, bool gate_first,
+                    c10::optional<torch::Tensor> floor_) {
+  TORCH_CHECK(o.is_cuda() && o.dtype() == torch::kFloat32 &&
+              o.is_contiguous() && o.dim() == 3);
+  const int T = o.size(0), H = o.size(1), PP = o.size(2);
+  const int P = floor_.has_value() ? PP - 1 : PP;
+  const int C = H * P;
+  TORCH_CHECK(P >= 1 && group >= 1 && C % group == 0,
+              "norm groups must divide the channels");
+  TORCH_CHECK(out.is_contiguous() && out.size(0) == T && out.size(1) == C);
+  TORCH_CHECK(gate.dim() == 2 && gate.stride(1) == 1 && gate.size(0) == T &&
+              gate.size(1) == C && gate.dtype() == out.dtype());
+  TORCH_CHECK(w.dtype() == torch::kFloat32 && w.numel() == C &&
+              w.is_contiguous());
+  if (floor_.has_value())
+    TORCH_CHECK(floor_->dtype() == torch::kFloat32 &&
+                floor_->is_contiguous() && floor_->numel() == (int64_t)T * H);
+  if (T == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  IGW_DISPATCH_ACT(out, {
+    hipLaunchKernelGGL(
+        (head_norm_gate_kernel<act_t>), dim3(C / group, T), dim3(64), 0,
+        stream, (act_t*)out.data_ptr(), (const float*)o.data_ptr(),
+        (const act_t*)gate.data_ptr(), (int64_t)gate.stride(0),
+        (const float*)w.data_ptr(),
+        floor_.has_value() ? (const float*)floor_->data_ptr() : nullptr, H, P,
+        PP, (int)group, (float)eps, gate_act == 1 ? 1 : 0,
+        gate_first ? 1 : 0);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------------------------------
+// paged append, keys and values of unequal width
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void append_paged_kv_kernel(
+    const T* __restrict__ k, int64_t k_stride, const T* __restrict__ v,
+    int64_t v_stride, T* __restrict__ kcache, T* __restrict__ vcache,
+    const int32_t* __restrict__ slot_mapping, int G, int N, int P,
+    int block_size) {
+  const int t = blockIdx.x;
+  const int slot = slot_mapping[t];
+  const int64_t blk = slot / block_size, off = slot % block_size;
+  for (int i = threadIdx.x; i < G * N; i += 256) {
+    const int g = i / N, n = i % N;
+    kcache[((blk * G + g) * block_size + off) * N + n] = k[t * k_stride + i];
+  }
+  for (int i = threadIdx.x; i < G * P; i += 256) {
+    const int g = i / P, p = i % P;
+    vcache[((blk * G + g) * block_size + off) * P + p] = v[t * v_stride + i];
+  }
+}
+
+void append_paged_kv(torch::Tensor k, torch::Tensor v, torch::Tensor kcache,
+                     torch::Tensor vcache, torch::Tensor slot_mapping) {
+  TORCH_CHECK(k.is_cuda() && k.dim() == 2 && k.stride(1) == 1 &&
+              v.dim() == 2 && v.stride(1) == 1 && k.dtype() == v.dtype());
+  TORCH_CHECK(kcache.is_contiguous() && vcache.is_contiguous() &&
+              kcache.dim() == 4 && vcache.dim() == 4 &&
+              kcache.dtype() == k.dtype() && vcache.dtype() == k.dtype());
+  const int T = k.size(0), G = kcache.size(1), bs = kcache.size(2);
+  const int N = kcache.size(3), P = vcache.size(3);
+  TORCH_CHECK(vcache.size(0) == kcache.size(0) && vcache.size(1) == G &&
+              vcache.size(2) == bs);
+  TORCH_CHECK(k.size(1) == G * N && v.size(1) == G * P && v.size(0) == T);
+  TORCH_CHECK(slot_mapping.dtype() == torch::kInt32 &&
+              slot_mapping.numel() == T);
+  if (T == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  IGW_DISPATCH_ACT(k, {
+    hipLaunchKernelGGL(
+        (append_paged_kv_kernel<act_t>), dim3(T), dim3(256), 0, stream,
+        (const act_t*)k.data_ptr(), (int64_t)k.stride(0),
+        (const act_t*)v.data_ptr(), (int64_t)v.stride(0),
+        (act_t*)kcache.data_ptr(), (act_t*)vcache.data_ptr(),
+        (const int32_t*)slot_mapping.data_ptr(), G, N, P, bs);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------------------------------------
+// average of two normed branches
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(RROW_BLOCK) void rmsnorm_pair_mean_kernel(
+    T* __restrict__ out, const T* __restrict__ a, const T* __restrict__ b,
+    const float* __restrict__ wa, const float* __restrict__ wb, int D,
+    float eps) {
+  __shared__ float lds[RROW_BLOCK / 64];
+  const int64_t row = blockIdx.x;
+  const T* ar = a + row * D;
+  const T* br = b + row * D;
+  float sa = 0.0f, sb = 0.0f;
+  for (int d = threadIdx.x; d < D; d += RROW_BLOCK) {
+    const float x = Act<T>::ld(ar + d), y = Act<T>::ld(br + d);
+    sa += x * x;
+    sb += y * y;
+  }
+  const float ra = 1.0f / sqrtf(rrow_block_sum(sa, lds) / (float)D + eps);
+  const float rb = 1.0f / sqrtf(rrow_block_sum(sb, lds) / (float)D + eps);
+  for (int d = threadIdx.x; d < D; d += RROW_BLOCK)
+    Act<T>::st(out + row * D + d,
+               0.5f * (Act<T>::ld(ar + d) * ra * wa[d] +
+                       Act<T>::ld(br + d) * rb * wb[d]));
+}
+
+void rmsnorm_pair_mean(torch::Tensor out, torch::Tensor a, torch::Tensor b,
+                       torch::Tensor wa, torch::Tensor wb, double eps) {
+  TORCH_CHECK(a.is_cuda() && a.is_contiguous() && b.is_contiguous() &&
+              a.dim() == 2 && a.sizes() == b.sizes() &&
+              a.dtype() == b.dtype());
+  const int T = a.size(0), D = a.size(1);
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == a.sizes() &&
+              out.dtype() == a.dtype());
+  TORCH_CHECK(wa.dtype() == torch::kFloat32 && wa.numel() == D &&
+              wb.dtype() == torch::kFloat32 && wb.numel() == D);
+  if (T == 0) return;
+  hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  IGW_DISPATCH_ACT(a, {
+    hipLaunchKernelGGL((rmsnorm_pair_mean_kernel<act_t>), dim3(T),
+                       dim3(RROW_BLOCK), 0, stream, (act_t*)out.data_ptr(),
+                       (const act_t*)a.data_ptr(), (const act_t*)b.data_ptr(),
+                       (const float*)wa.data_ptr(), (const float*)wb.data_ptr(),
+                       D, (float)eps);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+}  // namespace igw
