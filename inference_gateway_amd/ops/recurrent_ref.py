@@ -61,7 +61,8 @@ def causal_conv_ref(x, w, bias, state, seq_cu, seq_start, seq_slots, silu):
     for r0, r1, st, sl in _seqs(seq_cu, seq_start, seq_slots):
         if r1 == r0:
             continue
-        hist = (state[sl].view(taps - 1, C).clone() if st > 0 else
+        hist = (state[sl, :(taps - 1) * C].view(taps - 1, C).clone()
+                if st > 0 else
                 torch.zeros((taps - 1, C), dtype=torch.float32,
                             device=x.device))
         u = torch.cat([hist, xf[r0:r1]], 0)          # [taps-1 + n, C]

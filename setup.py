@@ -18,13 +18,20 @@ from torch.utils import cpp_extension  # noqa: E402
 ROOT = Path(__file__).parent
 CSRC = ROOT / "inference_gateway_amd" / "ops" / "csrc"
 
-sources = [str(CSRC / "bindings.cpp")] + sorted(
-    str(p) for p in CSRC.glob("*.hip")
-)
+def _hip_sources(d):
+    # hipify leaves shadow copies (x_hip.hip) beside the sources
+    return sorted(str(p) for p in d.glob("*.hip")
+                  if not p.name.endswith("_hip.hip"))
+
+
+sources = [str(CSRC / "bindings.cpp")] + _hip_sources(CSRC)
 HYB = ROOT / "inference_gateway_amd" / "ops" / "csrc_hybrid"
-hybrid_sources = [str(HYB / "bindings.cpp")] + sorted(
-    str(p) for p in HYB.glob("*.hip")
-)
+hybrid_sources = [str(HYB / "bindings.cpp")] + _hip_sources(HYB)
+
+REC = ROOT / "inference_gateway_amd" / "ops" / "csrc_recurrent"
+# the recurrent extension also compiles the two hybrid source files whose
+# row kernels (fused add + RMS norm, squared ReLU) its models share
+recurrent_sources = [str(REC / "bindings.cpp")] + _hip_sources(REC) + [str(HYB / "parallel_ops.hip"), str(HYB / "hybrid_ops.hip")]
 
 # packed-fp32 instruction selection is switched off for all device code
 HIPCC_FLAGS = [
@@ -44,8 +51,9 @@ def _ext(name, srcs):
     )
 
 
-# IGW_BUILD_EXT=hybrid|kernels builds just one extension (a process that
-# serves one model family compiles only what it loads); default: both
+# IGW_BUILD_EXT=hybrid|kernels|recurrent builds just one extension (a
+# process that serves one model family compiles only what it loads);
+# default: all
 _which = os.environ.get("IGW_BUILD_EXT", "all")
 ext_modules = []
 if _which in ("all", "kernels"):
@@ -53,6 +61,10 @@ if _which in ("all", "kernels"):
 if _which in ("all", "hybrid"):
     ext_modules.append(_ext("inference_gateway_amd.ops._hybrid",
                             hybrid_sources))
+
+if _which in ("all", "recurrent"):
+    ext_modules.append(_ext("inference_gateway_amd.ops._recurrent",
+                            recurrent_sources))
 
 setup(
     name="inference_gateway_amd_kernels",

@@ -92,9 +92,11 @@ def softcap_attention(q, k, v, H, G, scale, cap, coef, every):
 def left_mixer(h, W, pre, m):
     H, G, N, P = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     T = h.shape[0]
-    q = short_conv(h @ W[pre + "q"].T, W[pre + "q.conv"])
-    k = short_conv(h @ W[pre + "k"].T, W[pre + "k.conv"])
-    v = short_conv(h @ W[pre + "v"].T, W[pre + "v.conv"])
+    q, k, v = (h @ W[pre + c].T for c in "qkv")
+    if m.get("conv", 1) > 1:
+        q = short_conv(q, W[pre + "q.conv"])
+        k = short_conv(k, W[pre + "k.conv"])
+        v = short_conv(v, W[pre + "v.conv"])
     o = softcap_attention(q.reshape(T, H, N), k.reshape(T, G, N),
                           v.reshape(T, G, P), H, G, m["scale"],
                           m["softcap"], m["q_temp"]["coef"],
@@ -223,3 +225,147 @@ def forward(W, cfg, tokens):
         taps.append(x.copy())
     logits = norm_one_plus(x, W["final.norm"], eps) @ W["embed"].T
     return logits, np.stack(taps)
+
+
+# ---------------------------------------------------------------------------
+# random checkpoints for the tests
+# ---------------------------------------------------------------------------
+def tensor_shapes(cfg):
+    """Tensor name -> shape of a checkpoint of this configuration."""
+    D, V = cfg["width"], cfg["vocab"]
+    sh = {"embed": (V, D),
+          "bigram": (cfg["embedding"]["bigram"]["buckets"] + 1, D),
+          "pos": (cfg["max_positions"], D), "embed.norm": (D,),
+          "final.norm": (D,)}
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        sh[p + "norm1"] = (D,)
+        if l["type"] == "mlstm":
+            H, N, P = m["heads"], m["dim"], m["vdim"]
+            sh.update({p + "mix.q": (H * N, D), p + "mix.k": (H * N, D),
+                       p + "mix.v": (H * P, D), p + "mix.g": (H * P, D),
+                       p + "mix.o": (D, H * P), p + "mix.norm": (H * P,),
+                       p + "mix.i": (H, D), p + "mix.i.b": (H,),
+                       p + "mix.f": (H, D), p + "mix.f.b": (H,)})
+        elif l["type"] == "mamba2":
+            H, P, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
+            inner, cc = H * P, H * P + 2 * G * N
+            sh.update({p + "mix.in": (inner + cc + H, D),
+                       p + "mix.conv": (cc, m["conv"]),
+                       p + "mix.conv.b": (cc,), p + "mix.dt_bias": (H,),
+                       p + "mix.A_log": (H,), p + "mix.D": (H,),
+                       p + "mix.norm": (inner,), p + "mix.o": (D, inner)})
+        else:
+            a, b = m["left"], m["right"]
+            H, G, N, P = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            q = p + "mix.left."
+            sh.update({q + "q": (H * N, D), q + "k": (G * N, D),
+                       q + "v": (G * P, D), q + "o": (D, H * P),
+                       q + "out": (D,)})
+            if a["conv"] > 1:
+                sh.update({q + "q.conv": (H * N, a["conv"]),
+                           q + "k.conv": (G * N, a["conv"]),
+                           q + "v.conv": (G * P, a["conv"])})
+            r = p + "mix.right."
+            HN = b["heads"] * b["dim"]
+            R = b.get("decay_rank", 4)
+            sh.update({r + "mu." + s: (D,) for s in "rkvgw"})
+            sh.update({r + s: (HN, D) for s in "rkvg"})
+            sh.update({r + "w1": (R, D), r + "w2": (HN, R), r + "w0": (HN,),
+                       r + "u": (b["heads"], b["dim"]), r + "norm": (HN,),
+                       r + "o": (D, HN), r + "out": (D,)})
+        if l.get("mlp") is not None:
+            sh.update({p + "norm2": (D,), p + "mlp.up": (l["mlp"]["ff"], D),
+                       p + "mlp.down": (D, l["mlp"]["ff"])})
+    return sh
+
+
+def random_weights(cfg, seed=0):
+    """Random weights, rounded to bfloat16 (what a checkpoint stores),
+    as float64 arrays."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    W = {}
+    for name, shape in tensor_shapes(cfg).items():
+        x = torch.randn(shape, generator=g, dtype=torch.float32)
+        last = name.rsplit(".", 1)[-1]
+        if name in ("embed",):
+            x = x * 0.5 / cfg["embedding"]["scale"]
+        elif name in ("bigram", "pos"):
+            x = x * 0.5
+        elif last in ("norm1", "norm2") or name in ("embed.norm",
+                                                    "final.norm"):
+            x = x * 0.2                     # stored around zero
+        elif last in ("norm", "out", "D"):
+            x = 1.0 + x * 0.2
+        elif ".mu." in name:
+            x = torch.rand(shape, generator=g)
+        elif last == "w0":
+            x = -1.0 + x * 0.7
+        elif last in ("A_log", "dt_bias", "u"):
+            x = x * 0.5
+        elif name.endswith("f.b"):
+            x = 2.0 + x
+        elif name.endswith("i.b") or name.endswith("conv.b"):
+            x = x * 0.5
+        elif last == "conv":
+            x = x * 0.6
+        elif len(shape) == 2:
+            x = x * shape[1] ** -0.5 * (3.0 if last in ("i", "f", "w2")
+                                        else 1.0)
+        W[name] = x.to(torch.bfloat16).double().numpy()
+    return W
+
+
+def save_checkpoint(path, cfg, W):
+    """config.json + model.safetensors (bfloat16) in `path`."""
+    import json
+    import os
+
+    import torch
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: torch.from_numpy(v).to(torch.bfloat16).contiguous()
+               for k, v in W.items()},
+              os.path.join(path, "model.safetensors"))
+    return str(path)
+
+
+def make_config(width, vocab, layers, buckets=97, mul_prev=7, mul_cur=3,
+                scale=None, eps=1e-5, max_positions=700):
+    return {"architecture": "Feditar", "width": width, "vocab": vocab,
+            "max_positions": max_positions, "norm": {"eps": eps},
+            "embedding": {"scale": scale or float(width) ** 0.5,
+                          "bigram": {"buckets": buckets,
+                                     "mul_prev": mul_prev,
+                                     "mul_cur": mul_cur}},
+            "layers": layers}
+
+
+def mlstm_layer(heads, dim, vdim, cap=10.0, ff=0):
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim,
+                                       "vdim": vdim, "gate_cap": cap},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def mamba2_layer(heads, vdim, state, groups, conv, norm_groups, ff=0):
+    return {"type": "mamba2",
+            "mixer": {"heads": heads, "vdim": vdim, "state": state,
+                      "groups": groups, "conv": conv,
+                      "norm_groups": norm_groups},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def parallel_layer(heads, kv_heads, dim, vdim, conv, coef, every, scale,
+                   softcap, r_heads, r_dim, ff=0):
+    return {"type": "parallel",
+            "mixer": {"left": {"heads": heads, "kv_heads": kv_heads,
+                               "dim": dim, "vdim": vdim, "conv": conv,
+                               "q_temp": {"coef": coef, "every": every},
+                               "scale": scale, "softcap": softcap},
+                      "right": {"heads": r_heads, "dim": r_dim}},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
