@@ -85,8 +85,9 @@ def parse_args():
                          "tokens/s and per-kernel roofline fractions); "
                          "prints its own JSON object")
     ap.add_argument("--arch", type=str, default="fedatar",
-                    help="design for --arch-compare (fedatar | mekevik), "
-                         "each beside Mixtral")
+                    help="design for --arch-compare: fedatar or mekevik "
+                         "(each beside Mixtral) or feditar (beside "
+                         "Fedatar)")
     ap.add_argument("--arch-size", type=str, default="2k",
                     help="layer shape for --arch-compare (2k | 4k)")
     ap.add_argument("--num-gpu-blocks", type=int, default=0,
@@ -515,6 +516,8 @@ def main() -> None:
         sys.path.insert(0, str(Path(__file__).resolve().parent / "tools"))
         if args.arch == "mekevik":
             import bench_parallel as bench_hybrid
+        elif args.arch == "feditar":
+            import bench_recurrent as bench_hybrid
         else:
             import bench_hybrid
 

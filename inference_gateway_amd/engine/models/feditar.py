@@ -197,7 +197,7 @@ class SoftcapAttention(nn.Module):
         o = ops.softcap_attention(
             c[:, :HN], kc, vc, fb.seq_block_table, fb.row_seq, fb.positions,
             s.scale, s.softcap, s.temp_coef, s.temp_every, 0,
-            fb.num_chunk_rows, fb.seq_lens, fb.max_context)
+            fb.num_chunk_rows, fb.seq_lens, fb.seq_cu, fb.seq_start)
         return F.linear(o, self.o)
 
 

@@ -757,16 +757,33 @@ def append_paged_kv(k, v, kcache, vcache, slot_mapping):
 SOFTCAP_ATTENTION_MFMA = True
 
 
+@functools.lru_cache(maxsize=256)
+def _softcap_tiles(seq_lens: tuple, num_seqs: int, device):
+    """Tile map of the MFMA attention kernel: prompt portions (the first
+    len(seq_lens) sequences of the batch) cut into runs of its tile rows,
+    and the sequences that bring one decoded row.  Cached: serving
+    repeats the same batch shapes."""
+    tq = int(_recurrent.softcap_attention_tile_rows())
+    tseq, toff = torch_ref.make_prefill_tiles(seq_lens, tq, device)
+    dec = torch.arange(len(seq_lens), num_seqs, dtype=torch.int32,
+                       device=device)
+    return tseq, toff, dec
+
+
 def softcap_attention(q, kcache, vcache, block_table, row_seq, positions,
                       scale: float, softcap: float = 0.0,
                       temp_coef: float = 0.0, temp_every: int = 1,
                       window: int = 0, num_prefill_rows: int = 0,
-                      prefill_seq_lens=None, max_context: int = 0):
+                      prefill_seq_lens=None, seq_cu=None, seq_start=None):
     """Causal softmax attention over paged keys/values with grouped
     heads and separate key and value widths.  score = (q . k) * scale *
     (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)), squashed by
     softcap * tanh(. / softcap) when softcap > 0; window > 0 keeps the
-    last `window` keys.  q [T, H*N] (strided ok) -> [T, H*P]."""
+    last `window` keys.  q [T, H*N] (strided ok) -> [T, H*P].  Rows [0,
+    num_prefill_rows) are prompt portions (prefill_seq_lens = python row
+    counts of the first sequences), the rest single decoded tokens;
+    seq_cu / seq_start describe the sequences (needed by the tile
+    kernel; without them every batch runs the row kernel)."""
     if q.is_cuda:
         _require_recurrent()
         T = q.shape[0]
@@ -774,17 +791,14 @@ def softcap_attention(q, kcache, vcache, block_table, row_seq, positions,
         out = torch.empty((T, H * vcache.shape[3]), dtype=q.dtype,
                           device=q.device)
         if (q.dtype == torch.bfloat16 and SOFTCAP_ATTENTION_MFMA
-                and hasattr(_recurrent, "softcap_attention_mfma")):
-            tq = _recurrent.softcap_attention_tile_rows()
-            tiles = _attention_tiles(
-                tq, num_prefill_rows,
-                tuple(prefill_seq_lens or ()) if num_prefill_rows else (),
-                T, q.device)
+                and seq_cu is not None and seq_start is not None):
+            lens = tuple(prefill_seq_lens or ()) if num_prefill_rows else ()
+            tseq, toff, dec = _softcap_tiles(lens, seq_start.shape[0],
+                                             q.device)
             if _recurrent.softcap_attention_mfma(
-                    out, q, kcache, vcache, block_table, row_seq, positions,
-                    tiles[0], tiles[1], scale, softcap, temp_coef,
-                    temp_every, window, max_context or 4096,
-                    num_prefill_rows):
+                    out, q, kcache, vcache, block_table, seq_cu, seq_start,
+                    tseq, toff, dec, scale, softcap, temp_coef, temp_every,
+                    window):
                 return out
         _recurrent.softcap_attention(out, q, kcache, vcache, block_table,
                                      row_seq, positions, scale, softcap,

@@ -47,6 +47,14 @@ void softcap_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kcache,
                        torch::Tensor row_seq, torch::Tensor positions,
                        double scale, double softcap, double temp_coef,
                        int64_t temp_every, int64_t window);
+bool softcap_attention_mfma(torch::Tensor out, torch::Tensor q,
+                            torch::Tensor kcache, torch::Tensor vcache,
+                            torch::Tensor block_table, torch::Tensor seq_cu,
+                            torch::Tensor seq_start, torch::Tensor tile_seq,
+                            torch::Tensor tile_off, torch::Tensor dec_seq,
+                            double scale, double softcap, double temp_coef,
+                            int64_t temp_every, int64_t window);
+int64_t softcap_attention_tile_rows();
 // csrc_hybrid/parallel_ops.hip, csrc_hybrid/hybrid_ops.hip
 void add_rmsnorm_pair(torch::Tensor out1, c10::optional<torch::Tensor> out2,
                       torch::Tensor residual,
@@ -76,6 +84,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "outer-product memory recurrence, state columns in registers");
   m.def("softcap_attention", &igw::softcap_attention,
         "causal paged softmax attention with a tanh score cap");
+  m.def("softcap_attention_mfma", &igw::softcap_attention_mfma,
+        "capped softmax attention on MFMA tiles (bf16); false = sizes do "
+        "not fit, use softcap_attention");
+  m.def("softcap_attention_tile_rows", &igw::softcap_attention_tile_rows,
+        "query rows per MFMA tile");
   m.def("add_rmsnorm_pair", &igw::add_rmsnorm_pair,
         "fp32 residual += two deltas; one RMS statistic, two weighted outputs");
   m.def("relu2", &igw::relu2, "squared ReLU activation");

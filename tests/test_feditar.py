@@ -434,7 +434,7 @@ def _attention_case(device, dtype, H, G, N, P, bs, ctx, scale, cap, coef,
         q.reshape(ctx, -1).to(dtype).to(device), kc, vc,
         i32([perm], device), i32([0] * ctx, device),
         i32(list(range(ctx)), device), scale, cap, coef, every, 0, ctx,
-        [ctx], ctx)
+        [ctx], i32([0, ctx], device), i32([0], device))
     return out.float().cpu().numpy().reshape(ctx, H, P), ref
 
 
@@ -470,6 +470,58 @@ def test_attention_query_stretch_steps(device):
                               50.0, 0.0, 5)
     same = np.abs(out - base).reshape(40, -1).max(1) < 1e-6
     assert same[:4].all() and not same[4:].any()   # p + 1 >= 5 from row 4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dims", [
+    # H, G, N, P, page
+    (4, 2, 64, 64, 16), (9, 3, 88, 176, 16), (8, 2, 128, 128, 8),
+    (3, 1, 24, 72, 4), (2, 2, 40, 136, 16), (16, 1, 128, 64, 16)])
+def test_attention_tile_kernel_bf16(dims):
+    """The MFMA path over its padded instantiations: whole prompts
+    (several tiles, a ragged last one), then a mixed launch of a prompt
+    portion that continues a sequence beside decoded rows of others."""
+    H, G, N, P, bs = dims
+    dev = "cuda:0"
+    out, ref = _attention_case(dev, torch.bfloat16, H, G, N, P, bs, 150,
+                               N ** -0.5, 6.0, 0.4, 32)
+    assert np.abs(out - ref).max() < 0.06
+    out, ref = _attention_case(dev, torch.bfloat16, H, G, N, P, bs, 70,
+                               1.0, 9.0, 0.0, 1, boost=(69, 2, 4.0))
+    assert np.abs(out - ref).max() < 0.06
+    # three sequences of 90, 130 and 64 cached tokens: the first brings
+    # its last 37 rows as a portion, the others one decoded row each
+    g = torch.Generator().manual_seed(N + P)
+    lens, news = [90, 130, 64], [37, 1, 1]
+    qs, refs, slots, tables = [], [], [], []
+    nb = sum((L + bs - 1) // bs for L in lens)
+    kc = torch.zeros(nb + 2, G, bs, N, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros(nb + 2, G, bs, P, dtype=torch.bfloat16, device=dev)
+    perm = torch.randperm(nb + 2, generator=g).tolist()
+    maxb = max((L + bs - 1) // bs for L in lens)
+    for L, n in zip(lens, news):
+        q = torch.randn(L, H, N, generator=g).bfloat16().float()
+        k = torch.randn(L, G, N, generator=g).bfloat16().float()
+        v = torch.randn(L, G, P, generator=g).bfloat16().float()
+        r = oracle.softcap_attention(
+            q.double().numpy(), k.double().numpy(), v.double().numpy(), H,
+            G, N ** -0.5, 6.0, 0.4, 32)
+        mine = [perm.pop() for _ in range((L + bs - 1) // bs)]
+        tables.append(mine + [0] * (maxb - len(mine)))
+        sl = [mine[j // bs] * bs + j % bs for j in range(L)]
+        ops.append_paged_kv(k.reshape(L, -1).bfloat16().to(dev),
+                            v.reshape(L, -1).bfloat16().to(dev), kc, vc,
+                            i32(sl, dev))
+        qs.append(q[L - n:].reshape(n, -1))
+        refs.append(r[L - n:])
+    cu = [0, 37, 38, 39]
+    out = ops.softcap_attention(
+        torch.cat(qs).bfloat16().to(dev), kc, vc, i32(tables, dev),
+        i32([0] * 37 + [1, 2], dev),
+        i32(list(range(53, 90)) + [129, 63], dev), N ** -0.5, 6.0, 0.4, 32,
+        0, 37, [37], i32(cu, dev), i32([53, 129, 63], dev))
+    got = out.float().cpu().numpy().reshape(39, H, P)
+    assert np.abs(got - np.concatenate(refs)).max() < 0.06
 
 
 # ---------------------------------------------------------------------------
