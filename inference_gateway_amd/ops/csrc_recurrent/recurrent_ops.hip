@@ -162,6 +162,138 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   Act<T>::st(out + (int64_t)t * C + c, acc);
 }
 
+// 8 consecutive activations <-> 8 floats (16-byte accesses for bf16)
+template <typename T>
+struct Row8;
+template <>
+struct Row8<float> {
+  static DEVINLINE void ld(const float* p, float* o) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+  static DEVINLINE void st(float* p, const float* v) {
+    *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+    *(float4*)(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+template <>
+struct Row8<uint16_t> {
+  static DEVINLINE void ld(const uint16_t* p, float* o) {
+    const ushort8 r = *(const ushort8*)p;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = bf16_to_f32(r.v[e]);
+  }
+  static DEVINLINE void st(uint16_t* p, const float* v) {
+    ushort8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r.v[e] = f32_to_bf16(v[e]);
+    *(ushort8*)p = r;
+  }
+};
+
+// the same filter, one thread per (row, 8 channels): C % 8 == 0 and every
+// row 16-byte aligned
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_vec8_kernel(
+    T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
+    const float* __restrict__ w, const float* __restrict__ bias,
+    const float* __restrict__ state, const int32_t* __restrict__ seq_cu,
+    const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
+    int C, int taps, int silu) {
+  const int t = blockIdx.y;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (c >= C) return;
+  const int s = row_seq[t];
+  const int r0 = seq_cu[s];
+  const bool has_hist = seq_start[s] > 0;
+  const float* hist = state + (int64_t)seq_slots[s] * (taps - 1) * C;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = bias ? bias[c + e] : 0.0f;
+  for (int j = 0; j < taps; ++j) {
+    const int r = t - taps + 1 + j;
+    float u[8];
+    if (r >= r0) {
+      Row8<T>::ld(x + (int64_t)r * x_stride + c, u);
+    } else if (has_hist) {
+      Row8<float>::ld(hist + (int64_t)(taps - 1 - (r0 - r)) * C + c, u);
+    } else {
+      continue;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += w[(c + e) * taps + j] * u[e];
+  }
+  if (silu) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = silu_f32(acc[e]);
+  }
+  Row8<T>::st(out + (int64_t)t * C + c, acc);
+}
+
+// one thread per (ROWS consecutive rows, 8 channels), filter length known
+// at compile time: the rows' inputs and the filter are loaded once and
+// shared by the ROWS outputs
+template <typename T, int TAPS, int ROWS>
+__global__ __launch_bounds__(256) void causal_conv_tile_kernel(
+    T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
+    const float* __restrict__ w, const float* __restrict__ bias,
+    const float* __restrict__ state, const int32_t* __restrict__ seq_cu,
+    const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
+    int Trows, int C, int silu) {
+  const int t0 = blockIdx.y * ROWS;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (c >= C) return;
+  float wr[8][TAPS];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wr[e][j] = w[(c + e) * TAPS + j];
+  float xr[TAPS - 1 + ROWS][8];
+#pragma unroll
+  for (int k = 0; k < TAPS - 1 + ROWS; ++k) {
+    const int r = t0 - (TAPS - 1) + k;
+    if (r >= 0 && r < Trows) {
+      Row8<T>::ld(x + (int64_t)r * x_stride + c, xr[k]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xr[k][e] = 0.0f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) {
+    const int t = t0 + i;
+    if (t >= Trows) break;
+    const int s = row_seq[t];
+    const int r0 = seq_cu[s];
+    const bool has_hist = seq_start[s] > 0;
+    const float* hist = state + (int64_t)seq_slots[s] * (TAPS - 1) * C;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = bias ? bias[c + e] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+      const int r = t - TAPS + 1 + j;
+      if (r >= r0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += wr[e][j] * xr[i + j][e];
+      } else if (has_hist) {
+        float u[8];
+        Row8<float>::ld(hist + (int64_t)(TAPS - 1 - (r0 - r)) * C + c, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += wr[e][j] * u[e];
+      }
+    }
+    if (silu) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = silu_f32(acc[e]);
+    }
+    Row8<T>::st(out + (int64_t)t * C + c, acc);
+  }
+}
+
 // one thread per (sequence, channel): history <- last taps-1 inputs
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_kernel(
@@ -223,7 +355,37 @@ void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
               seq_slots.dtype() == torch::kInt32);
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  const bool vec8 =
+      C % 8 == 0 && (x.stride(0) * x.element_size()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(state.data_ptr()) % 16 == 0;
+#define LAUNCH_CONV_TILE(TP)                                                  \
+  hipLaunchKernelGGL(                                                        \
+      (causal_conv_tile_kernel<act_t, TP, 4>),                               \
+      dim3((C / 8 + 255) / 256, (T + 3) / 4), dim3(256), 0, stream,          \
+      (act_t*)out.data_ptr(), (const act_t*)x.data_ptr(),                    \
+      (int64_t)x.stride(0), (const float*)w.data_ptr(),                      \
+      bias.has_value() ? (const float*)bias->data_ptr() : nullptr,           \
+      (const float*)state.data_ptr(), (const int32_t*)seq_cu.data_ptr(),     \
+      (const int32_t*)seq_start.data_ptr(),                                  \
+      (const int32_t*)seq_slots.data_ptr(),                                  \
+      (const int32_t*)row_seq.data_ptr(), T, C, silu ? 1 : 0)
   IGW_DISPATCH_ACT(x, {
+    if (vec8 && taps == 4) LAUNCH_CONV_TILE(4);
+    else if (vec8 && taps == 3) LAUNCH_CONV_TILE(3);
+    else if (vec8 && taps == 2) LAUNCH_CONV_TILE(2);
+    else if (vec8)
+      hipLaunchKernelGGL(
+          (causal_conv_vec8_kernel<act_t>), dim3((C / 8 + 255) / 256, T),
+          dim3(256), 0, stream, (act_t*)out.data_ptr(),
+          (const act_t*)x.data_ptr(), (int64_t)x.stride(0),
+          (const float*)w.data_ptr(),
+          bias.has_value() ? (const float*)bias->data_ptr() : nullptr,
+          (const float*)state.data_ptr(), (const int32_t*)seq_cu.data_ptr(),
+          (const int32_t*)seq_start.data_ptr(),
+          (const int32_t*)seq_slots.data_ptr(),
+          (const int32_t*)row_seq.data_ptr(), C, taps, silu ? 1 : 0);
+    else
     hipLaunchKernelGGL(
         (causal_conv_kernel<act_t>), dim3((C + 255) / 256, T), dim3(256), 0,
         stream, (act_t*)out.data_ptr(), (const act_t*)x.data_ptr(),
@@ -241,6 +403,7 @@ void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
           (const int32_t*)seq_start.data_ptr(),
           (const int32_t*)seq_slots.data_ptr(), C, taps);
   });
+#undef LAUNCH_CONV_TILE
   HIP_CHECK_KERNEL();
 }
 
@@ -314,15 +477,18 @@ DEVINLINE float logsigmoid_f32(float x) {
   return fminf(x, 0.0f) - log1pf(expf(-fabsf(x)));
 }
 
-// one thread per (sequence, head), rows in order
+// One wave per (sequence, head), 64 rows per pass.  The recurrence m_t =
+// max(f_t + m_(t-1), i_t) is the composition of the maps m -> max(m + a, b)
+// with (a, b) = (f_t, i_t); composing (a1, b1) then (a2, b2) gives (a1 +
+// a2, max(b1 + a2, b2)), an associative operator, so the rows of a pass are
+// combined by a shuffle scan and m_t = max(m_start + A_t, B_t).  No
+// difference of large sums is ever formed.
 __global__ __launch_bounds__(64) void mlstm_gates_kernel(
     float* __restrict__ out, const float* __restrict__ pre,
     float* __restrict__ m_state, const int32_t* __restrict__ seq_cu,
     const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ seq_slots, int T, int H, int S, float cap) {
-  const int idx = blockIdx.x * 64 + threadIdx.x;
-  if (idx >= S * H) return;
-  const int s = idx / H, h = idx % H;
+  const int s = blockIdx.x / H, h = blockIdx.x % H, lane = threadIdx.x;
   const int r0 = seq_cu[s], r1 = seq_cu[s + 1];
   if (r1 == r0) return;
   float* ms = m_state + (int64_t)seq_slots[s] * H + h;
@@ -331,17 +497,35 @@ __global__ __launch_bounds__(64) void mlstm_gates_kernel(
   float* decay = out;
   float* kscale = out + (int64_t)T * H;
   float* floor_ = out + (int64_t)2 * T * H;
-  for (int t = r0; t < r1; ++t) {
-    const float gi = cap * tanhf(pre[(int64_t)t * 2 * H + h] * inv_cap);
-    const float gf =
-        logsigmoid_f32(cap * tanhf(pre[(int64_t)t * 2 * H + H + h] * inv_cap));
-    const float m_new = fmaxf(gf + m, gi);
-    decay[(int64_t)t * H + h] = expf(gf + m - m_new);
-    kscale[(int64_t)t * H + h] = expf(gi - m_new);
-    floor_[(int64_t)t * H + h] = expf(-m_new);
-    m = m_new;
+  for (int c0 = r0; c0 < r1; c0 += 64) {
+    const int t = c0 + lane;
+    const bool valid = t < r1;
+    float gi = -INFINITY, gf = 0.0f;
+    if (valid) {
+      gi = cap * tanhf(pre[(int64_t)t * 2 * H + h] * inv_cap);
+      gf = logsigmoid_f32(cap *
+                          tanhf(pre[(int64_t)t * 2 * H + H + h] * inv_cap));
+    }
+    float a = gf, b = gi;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const float pa = __shfl_up(a, off, 64), pb = __shfl_up(b, off, 64);
+      if (lane >= off) {
+        b = fmaxf(pb + a, b);
+        a = pa + a;
+      }
+    }
+    const float m_t = fmaxf(m + a, b);
+    float m_prev = __shfl_up(m_t, 1, 64);
+    if (lane == 0) m_prev = m;
+    if (valid) {
+      decay[(int64_t)t * H + h] = expf(gf + m_prev - m_t);
+      kscale[(int64_t)t * H + h] = expf(gi - m_t);
+      floor_[(int64_t)t * H + h] = expf(-m_t);
+    }
+    m = __shfl(m_t, min(63, r1 - c0 - 1), 64);
   }
-  *ms = m;
+  if (lane == 0) *ms = m;
 }
 
 void mlstm_gates(torch::Tensor out, torch::Tensor pre, double cap,
@@ -359,8 +543,7 @@ void mlstm_gates(torch::Tensor out, torch::Tensor pre, double cap,
               seq_slots.dtype() == torch::kInt32);
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
-  hipLaunchKernelGGL(mlstm_gates_kernel, dim3((S * H + 63) / 64), dim3(64), 0,
-                     stream, (float*)out.data_ptr(),
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(S * H), dim3(64), 0, stream, (float*)out.data_ptr(),
                      (const float*)pre.data_ptr(), (float*)m_state.data_ptr(),
                      (const int32_t*)seq_cu.data_ptr(),
                      (const int32_t*)seq_start.data_ptr(),
@@ -398,32 +581,53 @@ void ssm_gates(torch::Tensor out, torch::Tensor dt_pre, torch::Tensor a_log) {
 }
 
 // ---------------------------------------------------------------------------
-// read-out epilogue: one wave per (row, norm group)
+// read-out epilogue: a wave takes HNG_PAIRS consecutive (row, norm group)
+// pairs, four waves per workgroup
 // ---------------------------------------------------------------------------
+constexpr int HNG_PAIRS = 4;
+
 template <typename T>
-__global__ __launch_bounds__(64) void head_norm_gate_kernel(
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(
     T* __restrict__ out, const float* __restrict__ o,
     const T* __restrict__ gate, int64_t gate_stride,
     const float* __restrict__ w, const float* __restrict__ floor_, int H,
-    int P, int PP, int group, float eps, int gate_silu, int gate_first) {
-  const int t = blockIdx.y, g = blockIdx.x, lane = threadIdx.x;
+    int P, int PP, int group, float eps, int gate_silu, int gate_first,
+    int64_t npairs) {
+  const int lane = threadIdx.x & 63;
   const int C = H * P;
+  const int ng = C / group;
+  const int64_t first =
+      ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * HNG_PAIRS;
+  for (int64_t pair = first; pair < min(first + HNG_PAIRS, npairs); ++pair) {
+  const int t = (int)(pair / ng), g = (int)(pair % ng);
   const int c0 = g * group;
   const float* orow = o + (int64_t)t * H * PP;
   const T* grow = gate + (int64_t)t * gate_stride;
-  float sq = 0.0f;
-  // pass 1: the value before the norm, and its square sum
-  for (int i = lane; i < group; i += 64) {
+  // where channel c0 + i sits in o, without a division per element when
+  // the rows are dense (PP == P) or the group is one head
+  const bool dense = PP == P;
+  const bool one_head = group == P;
+  const int hg = one_head ? g : -1;
+  float inv_den_g = 1.0f;
+  if (floor_ != nullptr && one_head)
+    inv_den_g = 1.0f / (fmaxf(fabsf(orow[hg * PP + P]),
+                              floor_[(int64_t)t * H + hg]) + 1e-6f);
+  auto value = [&](int i) {
     const int c = c0 + i;
+    if (dense) return orow[c];
+    if (one_head) return orow[hg * PP + i] * inv_den_g;
     const int h = c / P, p = c % P;
     float v = orow[h * PP + p];
-    if (floor_ != nullptr) {
-      const float den =
-          fmaxf(fabsf(orow[h * PP + P]), floor_[(int64_t)t * H + h]) + 1e-6f;
-      v = v / den;
-    }
+    if (floor_ != nullptr)
+      v = v / (fmaxf(fabsf(orow[h * PP + P]), floor_[(int64_t)t * H + h]) +
+               1e-6f);
+    return v;
+  };
+  float sq = 0.0f;
+  for (int i = lane; i < group; i += 64) {
+    float v = value(i);
     if (gate_first) {
-      const float z = Act<T>::ld(grow + c);
+      const float z = Act<T>::ld(grow + c0 + i);
       v *= gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
     }
     sq += v * v;
@@ -431,19 +635,14 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(
   const float rstd = 1.0f / sqrtf(wave_reduce_sum(sq) / (float)group + eps);
   for (int i = lane; i < group; i += 64) {
     const int c = c0 + i;
-    const int h = c / P, p = c % P;
-    float v = orow[h * PP + p];
-    if (floor_ != nullptr) {
-      const float den =
-          fmaxf(fabsf(orow[h * PP + P]), floor_[(int64_t)t * H + h]) + 1e-6f;
-      v = v / den;
-    }
+    float v = value(i);
     const float z = Act<T>::ld(grow + c);
     const float gz = gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
     if (gate_first) v *= gz;
     v = v * rstd * w[c];
     if (!gate_first) v *= gz;
     Act<T>::st(out + (int64_t)t * C + c, v);
+  }
   }
 }
 
@@ -469,14 +668,16 @@ void head_norm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
   IGW_DISPATCH_ACT(out, {
+    const int64_t npairs = (int64_t)T * (C / group);
     hipLaunchKernelGGL(
-        (head_norm_gate_kernel<act_t>), dim3(C / group, T), dim3(64), 0,
+        (head_norm_gate_kernel<act_t>),
+        dim3((npairs + 4 * HNG_PAIRS - 1) / (4 * HNG_PAIRS)), dim3(256), 0,
         stream, (act_t*)out.data_ptr(), (const float*)o.data_ptr(),
         (const act_t*)gate.data_ptr(), (int64_t)gate.stride(0),
         (const float*)w.data_ptr(),
         floor_.has_value() ? (const float*)floor_->data_ptr() : nullptr, H, P,
         PP, (int)group, (float)eps, gate_act == 1 ? 1 : 0,
-        gate_first ? 1 : 0);
+        gate_first ? 1 : 0, npairs);
   });
   HIP_CHECK_KERNEL();
 }
@@ -503,6 +704,29 @@ __global__ __launch_bounds__(256) void append_paged_kv_kernel(
   }
 }
 
+// N % 8 == 0, P % 8 == 0, rows 16-byte aligned
+template <typename T>
+__global__ __launch_bounds__(256) void append_paged_kv_vec8_kernel(
+    const T* __restrict__ k, int64_t k_stride, const T* __restrict__ v,
+    int64_t v_stride, T* __restrict__ kcache, T* __restrict__ vcache,
+    const int32_t* __restrict__ slot_mapping, int G, int N, int P,
+    int block_size) {
+  const int t = blockIdx.x;
+  const int slot = slot_mapping[t];
+  const int64_t blk = slot / block_size, off = slot % block_size;
+  struct alignas(16) Vec { T v[8]; };
+  for (int i = threadIdx.x * 8; i < G * N; i += 256 * 8) {
+    const int g = i / N, n = i % N;
+    *(Vec*)(kcache + ((blk * G + g) * block_size + off) * N + n) =
+        *(const Vec*)(k + t * k_stride + i);
+  }
+  for (int i = threadIdx.x * 8; i < G * P; i += 256 * 8) {
+    const int g = i / P, p = i % P;
+    *(Vec*)(vcache + ((blk * G + g) * block_size + off) * P + p) =
+        *(const Vec*)(v + t * v_stride + i);
+  }
+}
+
 void append_paged_kv(torch::Tensor k, torch::Tensor v, torch::Tensor kcache,
                      torch::Tensor vcache, torch::Tensor slot_mapping) {
   TORCH_CHECK(k.is_cuda() && k.dim() == 2 && k.stride(1) == 1 &&
@@ -519,7 +743,21 @@ void append_paged_kv(torch::Tensor k, torch::Tensor v, torch::Tensor kcache,
               slot_mapping.numel() == T);
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  const int64_t es = k.element_size();
+  const bool vec8 = N % 8 == 0 && P % 8 == 0 &&
+                    (k.stride(0) * es) % 16 == 0 &&
+                    (v.stride(0) * es) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(k.data_ptr()) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(v.data_ptr()) % 16 == 0;
   IGW_DISPATCH_ACT(k, {
+    if (vec8)
+      hipLaunchKernelGGL(
+          (append_paged_kv_vec8_kernel<act_t>), dim3(T), dim3(256), 0, stream,
+          (const act_t*)k.data_ptr(), (int64_t)k.stride(0),
+          (const act_t*)v.data_ptr(), (int64_t)v.stride(0),
+          (act_t*)kcache.data_ptr(), (act_t*)vcache.data_ptr(),
+          (const int32_t*)slot_mapping.data_ptr(), G, N, P, bs);
+    else
     hipLaunchKernelGGL(
         (append_paged_kv_kernel<act_t>), dim3(T), dim3(256), 0, stream,
         (const act_t*)k.data_ptr(), (int64_t)k.stride(0),

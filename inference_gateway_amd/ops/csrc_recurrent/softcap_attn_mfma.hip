@@ -39,9 +39,10 @@ DEVINLINE float tanh_fast(float x) {
 
 constexpr int SA_BM = 64;
 constexpr int SA_BN = 64;
+constexpr int SA_BT_LDS = 1024;   // page numbers kept in LDS per sequence
 
 template <int NP, int PP, bool HEADS_ROWS>
-__global__ __launch_bounds__(256) void softcap_attention_mfma_kernel(
+__global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, int64_t q_rs,
     const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
     const int32_t* __restrict__ block_table, int max_blocks,
@@ -68,12 +69,19 @@ __global__ __launch_bounds__(256) void softcap_attention_mfma_kernel(
   const int rep = H / G;
   const int kvh = HEADS_ROWS ? blockIdx.y : blockIdx.y / rep;
   const int nrows = HEADS_ROWS ? rep : min(BM, Lq - qoff);  // valid rows
-  const int32_t* bt_row = block_table + (int64_t)seq * max_blocks;
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   uint16_t* pw_s = p_s + wave * 16 * BN;
+  // the sequence's page numbers sit in LDS when they fit, so that a K/V
+  // address does not wait on a second global load
+  __shared__ int32_t bt_s[SA_BT_LDS];
+  const int32_t* bt_row = block_table + (int64_t)seq * max_blocks;
+  const int nblk = (KVL + BS - 1) / BS;
+  if (nblk <= SA_BT_LDS) {
+    for (int i = tid; i < nblk; i += 256) bt_s[i] = bt_row[i];
+    bt_row = bt_s;      // visible after the barrier that follows Q staging
+  }
 
   // ---- Q tile -> LDS (the K region) -> A fragments ----
   for (int it = 0; it < BM * NP / 8 / 256; ++it) {
@@ -129,46 +137,67 @@ __global__ __launch_bounds__(256) void softcap_attention_mfma_kernel(
   const int kfirst =
       window > 0 ? max(0, P0 + qoff - window + 1) / BN * BN : 0;
 
-  for (int kbase = kfirst; kbase < kend; kbase += BN) {
-    __syncthreads();
-    for (int it = 0; it < BN * NP / 8 / 256; ++it) {
+  // the next K/V tile travels in registers while the current one is used
+  constexpr int KIT = BN * NP / 8 / 256, VIT = BN * PP / 8 / 256;
+  ushort8 kreg[KIT], vreg[VIT];
+  auto fetch = [&](int kbase) {
+#pragma unroll
+    for (int it = 0; it < KIT; ++it) {
       const int idx = tid + it * 256;
       const int row = idx / (NP / 8);
       const int d8 = (idx % (NP / 8)) * 8;
-      ushort8 val;
       if (d8 < N) {
         const int gpos = min(kbase + row, KVL - 1);
         const int64_t blk = bt_row[gpos / BS];
-        val = *reinterpret_cast<const ushort8*>(
+        kreg[it] = *reinterpret_cast<const ushort8*>(
             kcache + ((blk * G + kvh) * BS + (gpos % BS)) * N + d8);
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) val.v[e] = 0;
+        for (int e = 0; e < 8; ++e) kreg[it].v[e] = 0;
       }
-      *reinterpret_cast<ushort8*>(reinterpret_cast<char*>(k_s) + row * KROWB +
-                                  swz<KROWB>(row, d8 * 2)) = val;
     }
-    for (int it = 0; it < BN * PP / 8 / 256; ++it) {
+#pragma unroll
+    for (int it = 0; it < VIT; ++it) {
       const int idx = tid + it * 256;
       const int key = idx / (PP / 8);
       const int d8 = (idx % (PP / 8)) * 8;
-      ushort8 val;
       if (d8 < P) {
         const int gpos = min(kbase + key, KVL - 1);
         const int64_t blk = bt_row[gpos / BS];
-        val = *reinterpret_cast<const ushort8*>(
+        vreg[it] = *reinterpret_cast<const ushort8*>(
             vcache + ((blk * G + kvh) * BS + (gpos % BS)) * P + d8);
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) val.v[e] = 0;
+        for (int e = 0; e < 8; ++e) vreg[it].v[e] = 0;
       }
+    }
+  };
+  if (kfirst < kend) fetch(kfirst);
+
+  for (int kbase = kfirst; kbase < kend; kbase += BN) {
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < KIT; ++it) {
+      const int idx = tid + it * 256;
+      const int row = idx / (NP / 8);
+      const int d8 = (idx % (NP / 8)) * 8;
+      *reinterpret_cast<ushort8*>(reinterpret_cast<char*>(k_s) + row * KROWB +
+                                  swz<KROWB>(row, d8 * 2)) = kreg[it];
+    }
+#pragma unroll
+    for (int it = 0; it < VIT; ++it) {
+      const int idx = tid + it * 256;
+      const int key = idx / (PP / 8);
+      const int d8 = (idx % (PP / 8)) * 8;
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         *reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(vt_s) +
                                      (d8 + e) * (BN * 2) +
-                                     swz<128>(d8 + e, key * 2)) = val.v[e];
+                                     swz<128>(d8 + e, key * 2)) =
+            vreg[it].v[e];
     }
     __syncthreads();
+    if (kbase + BN < kend) fetch(kbase + BN);
 
     float4v acc_s[4];
 #pragma unroll

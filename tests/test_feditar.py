@@ -167,16 +167,16 @@ def test_embedding_pair_hash_and_slots(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("taps", [1, 2, 4, 5])
+@pytest.mark.parametrize("taps", [1, 2, 3, 4, 5])
 @pytest.mark.parametrize("silu", [False, True])
-def test_causal_conv_portions(device, taps, silu):
+@pytest.mark.parametrize("C", [70, 72])
+def test_causal_conv_portions(device, taps, silu, C):
     """Portions shorter than the filter, a one-row continuation and a
     fresh sequence over stale history; strided input rows."""
-    C = 70
     g = torch.Generator().manual_seed(taps)
     w = torch.randn(C, taps, generator=g)
     b = torch.randn(C, generator=g) if silu else None
-    full = [torch.randn(n, C + 3, generator=g) for n in (11, 6, 3)]
+    full = [torch.randn(n, C + 8, generator=g) for n in (11, 6, 3)]
     ref = []
     for x in full:
         y = oracle.short_conv(x[:, :C].double().numpy(), w.double().numpy(),
@@ -263,7 +263,8 @@ def _scan_reference(q, k, v, a, c, u, skip, ones, qscale):
     # H, G, N, P, form
     (2, 2, 6, 5, "mlstm"), (4, 2, 17, 3, "ssm"), (3, 3, 10, 10, "decay"),
     (2, 1, 33, 70, "mlstm"), (1, 1, 130, 65, "ssm"), (2, 2, 70, 70, "decay"),
-    (1, 1, 1, 1, "ssm")])
+    (1, 1, 1, 1, "ssm"), (2, 2, 8, 200, "mlstm"), (2, 1, 64, 300, "ssm"),
+    (2, 2, 32, 64, "decay"), (1, 1, 128, 16, "mlstm")])
 def test_outer_scan_forms(device, shape):
     """The three uses of the memory kernel, in two steps over a ragged
     batch: a fresh sequence in a stale slot, a continued one, a long one
