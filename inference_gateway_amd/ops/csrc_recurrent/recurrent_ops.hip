@@ -582,11 +582,13 @@ void ssm_gates(torch::Tensor out, torch::Tensor dt_pre, torch::Tensor a_log) {
 
 // ---------------------------------------------------------------------------
 // read-out epilogue: a wave takes HNG_PAIRS consecutive (row, norm group)
-// pairs, four waves per workgroup
+// pairs at once (all their loads are in flight together; the values wait
+// in registers between the statistic and the store), four waves per
+// workgroup.  VPL = values per lane: group <= 64 * VPL.
 // ---------------------------------------------------------------------------
 constexpr int HNG_PAIRS = 4;
 
-template <typename T>
+template <typename T, int VPL>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(
     T* __restrict__ out, const float* __restrict__ o,
     const T* __restrict__ gate, int64_t gate_stride,
@@ -598,24 +600,93 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(
   const int ng = C / group;
   const int64_t first =
       ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * HNG_PAIRS;
-  for (int64_t pair = first; pair < min(first + HNG_PAIRS, npairs); ++pair) {
-  const int t = (int)(pair / ng), g = (int)(pair % ng);
-  const int c0 = g * group;
-  const float* orow = o + (int64_t)t * H * PP;
-  const T* grow = gate + (int64_t)t * gate_stride;
   // where channel c0 + i sits in o, without a division per element when
   // the rows are dense (PP == P) or the group is one head
   const bool dense = PP == P;
   const bool one_head = group == P;
-  const int hg = one_head ? g : -1;
-  float inv_den_g = 1.0f;
-  if (floor_ != nullptr && one_head)
-    inv_den_g = 1.0f / (fmaxf(fabsf(orow[hg * PP + P]),
-                              floor_[(int64_t)t * H + hg]) + 1e-6f);
+  float val[HNG_PAIRS][VPL], gz[HNG_PAIRS][VPL], inv_den[HNG_PAIRS];
+#pragma unroll
+  for (int j = 0; j < HNG_PAIRS; ++j) {
+    const int64_t pair = min(first + j, npairs - 1);
+    const int t = (int)(pair / ng), g = (int)(pair % ng);
+    const int c0 = g * group;
+    const float* orow = o + (int64_t)t * H * PP;
+    const T* grow = gate + (int64_t)t * gate_stride;
+    inv_den[j] = 1.0f;
+    if (floor_ != nullptr && one_head)
+      inv_den[j] = 1.0f / (fmaxf(fabsf(orow[g * PP + P]),
+                                 floor_[(int64_t)t * H + g]) + 1e-6f);
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) {
+      const int i = lane + 64 * e;
+      float v = 0.0f, z = 0.0f;
+      if (i < group) {
+        const int c = c0 + i;
+        if (dense) {
+          v = orow[c];
+        } else if (one_head) {
+          v = orow[g * PP + i];
+        } else {
+          const int h = c / P, p = c % P;
+          v = orow[h * PP + p];
+          if (floor_ != nullptr)
+            v = v / (fmaxf(fabsf(orow[h * PP + P]),
+                           floor_[(int64_t)t * H + h]) + 1e-6f);
+        }
+        z = Act<T>::ld(grow + c);
+      }
+      val[j][e] = v;
+      gz[j][e] = z;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < HNG_PAIRS; ++j) {
+    float sq = 0.0f;
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) {
+      const float z = gz[j][e];
+      const float a = gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
+      float v = val[j][e] * inv_den[j];
+      if (gate_first) v *= a;
+      gz[j][e] = a;
+      val[j][e] = v;
+      if (lane + 64 * e < group) sq += v * v;
+    }
+    const float rstd = 1.0f / sqrtf(wave_reduce_sum(sq) / (float)group + eps);
+    const int64_t pair = first + j;
+    if (pair >= npairs) continue;
+    const int t = (int)(pair / ng), c0 = (int)(pair % ng) * group;
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) {
+      const int i = lane + 64 * e;
+      if (i >= group) continue;
+      float v = val[j][e] * rstd * w[c0 + i];
+      if (!gate_first) v *= gz[j][e];
+      Act<T>::st(out + (int64_t)t * C + c0 + i, v);
+    }
+  }
+}
+
+// any group size: one (row, group) pair per wave at a time, two passes
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(
+    T* __restrict__ out, const float* __restrict__ o,
+    const T* __restrict__ gate, int64_t gate_stride,
+    const float* __restrict__ w, const float* __restrict__ floor_, int H,
+    int P, int PP, int group, float eps, int gate_silu, int gate_first,
+    int64_t npairs) {
+  const int lane = threadIdx.x & 63;
+  const int C = H * P;
+  const int ng = C / group;
+  const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= npairs) return;
+  const int t = (int)(pair / ng), g = (int)(pair % ng);
+  const int c0 = g * group;
+  const float* orow = o + (int64_t)t * H * PP;
+  const T* grow = gate + (int64_t)t * gate_stride;
   auto value = [&](int i) {
     const int c = c0 + i;
-    if (dense) return orow[c];
-    if (one_head) return orow[hg * PP + i] * inv_den_g;
+    if (PP == P) return orow[c];
     const int h = c / P, p = c % P;
     float v = orow[h * PP + p];
     if (floor_ != nullptr)
@@ -637,12 +708,11 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(
     const int c = c0 + i;
     float v = value(i);
     const float z = Act<T>::ld(grow + c);
-    const float gz = gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
-    if (gate_first) v *= gz;
+    const float gzv = gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
+    if (gate_first) v *= gzv;
     v = v * rstd * w[c];
-    if (!gate_first) v *= gz;
+    if (!gate_first) v *= gzv;
     Act<T>::st(out + (int64_t)t * C + c, v);
-  }
   }
 }
 
@@ -667,18 +737,30 @@ void head_norm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
                 floor_->is_contiguous() && floor_->numel() == (int64_t)T * H);
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  const int64_t npairs = (int64_t)T * (C / group);
+#define HNG_ARGS                                                              \
+  (act_t*)out.data_ptr(), (const float*)o.data_ptr(),                         \
+      (const act_t*)gate.data_ptr(), (int64_t)gate.stride(0),                 \
+      (const float*)w.data_ptr(),                                             \
+      floor_.has_value() ? (const float*)floor_->data_ptr() : nullptr, H, P,  \
+      PP, (int)group, (float)eps, gate_act == 1 ? 1 : 0, gate_first ? 1 : 0,  \
+      npairs
+#define LAUNCH_HNG(VPL)                                                       \
+  hipLaunchKernelGGL((head_norm_gate_kernel<act_t, VPL>),                     \
+                     dim3((npairs + 4 * HNG_PAIRS - 1) / (4 * HNG_PAIRS)),    \
+                     dim3(256), 0, stream, HNG_ARGS)
   IGW_DISPATCH_ACT(out, {
-    const int64_t npairs = (int64_t)T * (C / group);
-    hipLaunchKernelGGL(
-        (head_norm_gate_kernel<act_t>),
-        dim3((npairs + 4 * HNG_PAIRS - 1) / (4 * HNG_PAIRS)), dim3(256), 0,
-        stream, (act_t*)out.data_ptr(), (const float*)o.data_ptr(),
-        (const act_t*)gate.data_ptr(), (int64_t)gate.stride(0),
-        (const float*)w.data_ptr(),
-        floor_.has_value() ? (const float*)floor_->data_ptr() : nullptr, H, P,
-        PP, (int)group, (float)eps, gate_act == 1 ? 1 : 0,
-        gate_first ? 1 : 0, npairs);
+    if (group <= 64) LAUNCH_HNG(1);
+    else if (group <= 128) LAUNCH_HNG(2);
+    else if (group <= 256) LAUNCH_HNG(4);
+    else if (group <= 512) LAUNCH_HNG(8);
+    else
+      hipLaunchKernelGGL((head_norm_gate_wide_kernel<act_t>),
+                         dim3((npairs + 3) / 4), dim3(256), 0, stream,
+                         HNG_ARGS);
   });
+#undef LAUNCH_HNG
+#undef HNG_ARGS
   HIP_CHECK_KERNEL();
 }
 

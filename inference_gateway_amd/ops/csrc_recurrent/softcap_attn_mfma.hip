@@ -33,6 +33,14 @@ DEVINLINE int swz(int row, int colbyte) {
   return colbyte ^ ((row & (ROWB >= 256 ? 15 : 7)) << 4);
 }
 
+// The transposed V tile (rows = value entries, 128 bytes of keys each) is
+// WRITTEN by lanes whose rows differ by multiples of 8 and READ by lanes on
+// 16 consecutive rows; folding both the low and the next three row bits
+// into the 16-byte chunk index keeps either access to two lanes per bank.
+DEVINLINE int swz_vt(int row, int colbyte) {
+  return colbyte ^ ((((row & 7) ^ ((row >> 3) & 7))) << 4);
+}
+
 DEVINLINE float tanh_fast(float x) {
   return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * x));
 }
@@ -193,7 +201,7 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
       for (int e = 0; e < 8; ++e)
         *reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(vt_s) +
                                      (d8 + e) * (BN * 2) +
-                                     swz<128>(d8 + e, key * 2)) =
+                                     swz_vt(d8 + e, key * 2)) =
             vreg[it].v[e];
     }
     __syncthreads();
@@ -265,7 +273,7 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
         const int vrow = nt * 16 + frag_m;
         short8v vfrag = *reinterpret_cast<const short8v*>(
             reinterpret_cast<char*>(vt_s) + vrow * (BN * 2) +
-            swz<128>(vrow, (kk2 * 32 + frag_k8) * 2));
+            swz_vt(vrow, (kk2 * 32 + frag_k8) * 2));
         acc_o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pfrag, vfrag,
                                                             acc_o[nt], 0, 0, 0);
       }

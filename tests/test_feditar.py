@@ -384,6 +384,32 @@ def test_head_norm_gate_modes(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dims", [(3, 5, 130, 650), (2, 4, 96, 384),
+                                  (4, 3, 70, 70)])
+def test_head_norm_gate_group_sizes(device, dims):
+    """Groups from one head to several, up to the two-pass kernel."""
+    T, H, P, group = dims
+    g = torch.Generator().manual_seed(P)
+    o = torch.randn(T, H, P, generator=g)
+    gate = torch.randn(T, H * P, generator=g)
+    w = torch.randn(H * P, generator=g)
+    for first in (True, False):
+        y = o.double().numpy().reshape(T, -1)
+        a = oracle.silu(gate.double().numpy())
+        if first:
+            y = y * a
+        y = oracle.rms_unit(y.reshape(T, -1, group), 1e-6).reshape(T, -1) \
+            * w.double().numpy()
+        if not first:
+            y = y * a
+        got = ops.head_norm_gate(o.to(device), gate.to(device),
+                                 w.to(device), 1e-6, group, ops.GATE_SILU,
+                                 first, None, torch.float32)
+        np.testing.assert_allclose(got.cpu().numpy(), y, atol=3e-5,
+                                   rtol=3e-5)
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_rmsnorm_pair_mean_and_ssm_gates(device):
     g = torch.Generator().manual_seed(8)
     a, b = torch.randn(6, 50, generator=g) * 4, torch.randn(6, 50,
