@@ -542,15 +542,20 @@ class FeditarConfig:
             layers.append(LayerSpec(type=t, mixer=mixer, mlp=mlp))
         e = cfg.get("embedding") or {}
         bg = e.get("bigram") or {}
+        # table sizes the json leaves out come from the tensors
+        pos_rows = cfg.get("max_positions") or (
+            shapes["pos"][0] if "pos" in shapes else 2048)
+        buckets = bg.get("buckets") or (
+            shapes["bigram"][0] - 1 if "bigram" in shapes else 1)
         return FeditarConfig(
             name=name, hidden_size=int(cfg["width"]),
             vocab_size=int(cfg["vocab"]), layers=layers,
             norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-6)),
             embed_scale=float(e.get("scale", 1.0)),
-            pair_hash=PairHashSpec(buckets=int(bg.get("buckets", 1)),
+            pair_hash=PairHashSpec(buckets=int(buckets),
                                    mul_prev=int(bg.get("mul_prev", 1)),
                                    mul_cur=int(bg.get("mul_cur", 1))),
-            max_position=int(cfg.get("max_positions", 2048)))
+            max_position=int(pos_rows))
 
 
 def feditar_preset(name: str, width: int, vocab: int, pattern: str,

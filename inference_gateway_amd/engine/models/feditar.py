@@ -87,7 +87,7 @@ class MLSTMMixer(nn.Module):
         pre = F.linear(h.float(), self.gates_w, self.gates_b)
         decay, kscale, floor = ops.mlstm_gates(
             pre, s.gate_cap, m_state, fb.seq_cu, fb.seq_start, fb.seq_slots)
-        o = ops.outer_scan(
+        o, den = ops.outer_scan(
             proj[:, :H * N].view(T, H, N),
             proj[:, H * N:2 * H * N].view(T, H, N),
             proj[:, 2 * H * N:2 * H * N + H * P].view(T, H, P),
@@ -95,8 +95,8 @@ class MLSTMMixer(nn.Module):
             fb.seq_start, fb.seq_slots, fb.seq_rows, ops.DECAY_LINEAR,
             True, float(N) ** -0.5)
         y = ops.head_norm_gate(o, proj[:, 2 * H * N + H * P:], self.norm_w,
-                               self.eps, P, ops.GATE_SIGMOID, False, floor,
-                               self.dtype)
+                               self.eps, P, ops.GATE_SIGMOID, False, den,
+                               floor, self.dtype)
         return F.linear(y, self.o)
 
 
@@ -147,7 +147,7 @@ class Mamba2Mixer(nn.Module):
         xbc = ops.causal_conv(proj[:, inner:], self.conv_w, self.conv_b,
                               conv_state, fb.seq_cu, fb.seq_start,
                               fb.seq_slots, fb.row_seq, True)
-        o = ops.outer_scan(
+        o, _ = ops.outer_scan(
             xbc[:, inner + G * N:].view(T, G, N),
             xbc[:, inner:inner + G * N].view(T, G, N),
             xbc[:, :inner].view(T, H, P), decay.unsqueeze(-1), dt, None,
@@ -155,7 +155,7 @@ class Mamba2Mixer(nn.Module):
             fb.seq_rows, ops.DECAY_LINEAR, False, 1.0)
         y = ops.head_norm_gate(o, proj[:, :inner], self.norm_w, self.eps,
                                inner // s.norm_groups, ops.GATE_SILU, True,
-                               None, self.dtype)
+                               None, None, self.dtype)
         return F.linear(y, self.o)
 
 
@@ -246,13 +246,13 @@ class DecayMemory(nn.Module):
         rkvg = torch.bmm(mixes[:4], self.rkvg_t)          # [4, T, H*N]
         lw = F.linear(torch.tanh(F.linear(mixes[4].float(), self.w1)),
                       self.w2, self.w0)                    # fp32 [T, H*N]
-        o = ops.outer_scan(
+        o, _ = ops.outer_scan(
             rkvg[0].view(T, H, N), rkvg[1].view(T, H, N),
             rkvg[2].view(T, H, N), lw.view(T, H, N), None, self.bonus, None,
             mem, fb.seq_cu, fb.seq_start, fb.seq_slots, fb.seq_rows,
             ops.DECAY_EXP_NEG_EXP, False, 1.0)
         y = ops.head_norm_gate(o, rkvg[3], self.norm_w, self.eps, N,
-                               ops.GATE_SILU, False, None, self.dtype)
+                               ops.GATE_SILU, False, None, None, self.dtype)
         return F.linear(y, self.o)
 
 

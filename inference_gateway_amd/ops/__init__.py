@@ -706,40 +706,43 @@ def outer_scan(q, k, v, decay, kscale, bonus, skip, state, seq_cu,
     o_t = (S + diag(u) k_t v_t^T)^T q_t; o_t = o_t * qscale + skip_h v_t.
     q, k [T, G, N] (strided ok; head h reads group h // (H/G)), v [T, H,
     P], decay fp32 [T, H, 1 | N] holding a_t (DECAY_LINEAR) or x with a_t
-    = exp(-exp(x)) (DECAY_EXP_NEG_EXP); ones_col appends a column of ones
-    to v (PP = P + 1: the memory's normaliser).  Returns fp32 [T, H, PP].
-    seq_rows: python row counts (host side, picks the launch shape)."""
+    = exp(-exp(x)) (DECAY_EXP_NEG_EXP).  ones_col keeps one more memory
+    column fed with ones (PP = P + 1: the normaliser n_t = a n + c k).
+    Returns (o fp32 [T, H, P], n_t . q_t * qscale fp32 [T, H] or None).
+    seq_rows: python row counts (host side)."""
     if v.is_cuda:
         _require_recurrent()
         T, H, P = v.shape
-        out = torch.empty((T, H, P + (1 if ones_col else 0)),
-                          dtype=torch.float32, device=v.device)
-        _recurrent.outer_scan(out, q, k, v, decay, kscale, bonus, skip,
-                              state, seq_cu, seq_start, seq_slots,
+        out = torch.empty((T, H, P), dtype=torch.float32, device=v.device)
+        norm = (torch.empty((T, H), dtype=torch.float32, device=v.device)
+                if ones_col else None)
+        _recurrent.outer_scan(out, norm, q, k, v, decay, kscale, bonus,
+                              skip, state, seq_cu, seq_start, seq_slots,
                               decay_mode, ones_col, qscale)
-        return out
+        return out, norm
     return recurrent_ref.outer_scan_ref(
         q, k, v, decay, kscale, bonus, skip, state, seq_cu, seq_start,
         seq_slots, decay_mode, ones_col, qscale)
 
 
 def head_norm_gate(o, gate, w, eps: float, group: int, gate_act: int,
-                   gate_first: bool, floor, out_dtype):
-    """Epilogue of a memory read-out o fp32 [T, H, PP]: optional division
-    by max(|last column|, floor) + 1e-6 (floor [T, H] fp32), RMS norm in
-    groups of `group` channels times w [C] fp32, and a sigmoid or silu
-    gate from pre-activations gate [T, C] (strided ok) applied before or
-    after the norm.  Returns [T, C] in out_dtype."""
+                   gate_first: bool, den, floor, out_dtype):
+    """Epilogue of a memory read-out o fp32 [T, H, P]: optional division
+    of every head by max(|den|, floor) + 1e-6 (den, floor [T, H] fp32;
+    floor None = 0), RMS norm in groups of `group` channels times w [C]
+    fp32, and a sigmoid or silu gate from pre-activations gate [T, C]
+    (strided ok) applied before or after the norm.  Returns [T, C] in
+    out_dtype."""
     if o.is_cuda:
         _require_recurrent()
-        T, H, PP = o.shape
-        C = H * (PP - (1 if floor is not None else 0))
-        out = torch.empty((T, C), dtype=out_dtype, device=o.device)
+        T, H, P = o.shape
+        out = torch.empty((T, H * P), dtype=out_dtype, device=o.device)
         _recurrent.head_norm_gate(out, o, gate, w, eps, group, gate_act,
-                                  gate_first, floor)
+                                  gate_first, den, floor)
         return out
     return recurrent_ref.head_norm_gate_ref(o, gate, w, eps, group, gate_act,
-                                            gate_first, floor, out_dtype)
+                                            gate_first, den, floor,
+                                            out_dtype)
 
 
 def append_paged_kv(k, v, kcache, vcache, slot_mapping):

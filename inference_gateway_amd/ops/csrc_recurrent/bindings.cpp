@@ -29,12 +29,14 @@ void ssm_gates(torch::Tensor out, torch::Tensor dt_pre, torch::Tensor a_log);
 void head_norm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
                     torch::Tensor w, double eps, int64_t group,
                     int64_t gate_act, bool gate_first,
+                    c10::optional<torch::Tensor> den,
                     c10::optional<torch::Tensor> floor_);
 void append_paged_kv(torch::Tensor k, torch::Tensor v, torch::Tensor kcache,
                      torch::Tensor vcache, torch::Tensor slot_mapping);
 void rmsnorm_pair_mean(torch::Tensor out, torch::Tensor a, torch::Tensor b,
                        torch::Tensor wa, torch::Tensor wb, double eps);
-void outer_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
+void outer_scan(torch::Tensor out, c10::optional<torch::Tensor> norm_out,
+                torch::Tensor q, torch::Tensor k,
                 torch::Tensor v, torch::Tensor decay,
                 c10::optional<torch::Tensor> kscale,
                 c10::optional<torch::Tensor> bonus,

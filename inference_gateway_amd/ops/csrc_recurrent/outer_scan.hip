@@ -10,7 +10,7 @@
 // a_t is a scalar per head (VEC_DECAY = false) or one factor per key entry,
 // given either directly or as x with a = exp(-exp(x)).  With ones_col the
 // memory has one more column fed with v = 1 (the normaliser n_t = a n +
-// c k, read out as n_t . q_t).
+// c k); its read-out n_t . q_t goes to a tensor of its own.
 //
 // One workgroup per (run of value tiles, head, sequence); each of its up to
 // four waves takes 64 value columns, and a lane owns ONE column of S in
@@ -52,7 +52,8 @@ constexpr int SCAN_MAX_WAVES = 4;
 
 template <typename T, int NMAX, bool VEC_DECAY, bool BONUS, bool VEC8>
 __global__ __launch_bounds__(64 * SCAN_MAX_WAVES) void outer_scan_kernel(
-    float* __restrict__ out, const T* __restrict__ q, int64_t q_s0,
+    float* __restrict__ out, float* __restrict__ norm_out,
+    const T* __restrict__ q, int64_t q_s0,
     int64_t q_s1, const T* __restrict__ k, int64_t k_s0, int64_t k_s1,
     const T* __restrict__ v, int64_t v_s0, int64_t v_s1,
     const float* __restrict__ decay, const float* __restrict__ kscale,
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(64 * SCAN_MAX_WAVES) void outer_scan_kernel(
         }
         dot = wave_reduce_sum(dot);
         if (lane == 0)
-          out[((int64_t)(c0 + t) * H + h) * PP + P] = dot * qscale;
+          norm_out[(int64_t)(c0 + t) * H + h] = dot * qscale;
       }
     }
     if (BONUS) {
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(64 * SCAN_MAX_WAVES) void outer_scan_kernel(
           }
         }
       }
-      if (active) out[(row * H + h) * PP + p] = o * qscale + sk * vv;
+      if (active) out[(row * H + h) * P + p] = o * qscale + sk * vv;
     }
   }
   if (active) {
@@ -238,7 +239,8 @@ __global__ __launch_bounds__(64 * SCAN_MAX_WAVES) void outer_scan_kernel(
   }
 }
 
-void outer_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
+void outer_scan(torch::Tensor out, c10::optional<torch::Tensor> norm_out,
+                torch::Tensor q, torch::Tensor k,
                 torch::Tensor v, torch::Tensor decay,
                 c10::optional<torch::Tensor> kscale,
                 c10::optional<torch::Tensor> bonus,
@@ -256,7 +258,13 @@ void outer_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
   const int PP = P + (ones_col ? 1 : 0);
   TORCH_CHECK(q.size(0) == T && G >= 1 && H % G == 0);
   TORCH_CHECK(out.dtype() == torch::kFloat32 && out.is_contiguous() &&
-              out.numel() == (int64_t)T * H * PP);
+              out.numel() == (int64_t)T * H * P);
+  TORCH_CHECK(norm_out.has_value() == ones_col,
+              "the normaliser read-out goes with the ones column");
+  if (ones_col)
+    TORCH_CHECK(norm_out->dtype() == torch::kFloat32 &&
+                norm_out->is_contiguous() &&
+                norm_out->numel() == (int64_t)T * H);
   TORCH_CHECK(decay.dtype() == torch::kFloat32 && decay.is_contiguous() &&
               decay.dim() == 3 && decay.size(0) == T && decay.size(1) == H &&
               (decay.size(2) == 1 || decay.size(2) == N));
@@ -296,7 +304,9 @@ void outer_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
 #define LAUNCH_SCAN_V(NM, VD, BO, V8)                                         \
   hipLaunchKernelGGL(                                                         \
       (outer_scan_kernel<act_t, NM, VD, BO, V8>), grid, block, 0, stream,     \
-      (float*)out.data_ptr(), (const act_t*)q.data_ptr(),                     \
+      (float*)out.data_ptr(),                                                 \
+      ones_col ? (float*)norm_out->data_ptr() : nullptr,                      \
+      (const act_t*)q.data_ptr(),                                             \
       (int64_t)q.stride(0), (int64_t)q.stride(1),                             \
       (const act_t*)k.data_ptr(), (int64_t)k.stride(0),                       \
       (int64_t)k.stride(1), (const act_t*)v.data_ptr(),                       \

@@ -36,6 +36,31 @@ DEVINLINE float rrow_block_sum(float x, float* lds) {
 
 DEVINLINE float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
+// 4 consecutive activations <-> 4 floats
+template <typename T>
+struct Val4;
+template <>
+struct Val4<float> {
+  static DEVINLINE float4 ld(const float* p) { return *(const float4*)p; }
+  static DEVINLINE void st(float* p, float4 v) { *(float4*)p = v; }
+};
+template <>
+struct Val4<uint16_t> {
+  static DEVINLINE float4 ld(const uint16_t* p) {
+    const ushort4x r = *(const ushort4x*)p;
+    return make_float4(bf16_to_f32(r.v[0]), bf16_to_f32(r.v[1]),
+                       bf16_to_f32(r.v[2]), bf16_to_f32(r.v[3]));
+  }
+  static DEVINLINE void st(uint16_t* p, float4 v) {
+    ushort4x r;
+    r.v[0] = f32_to_bf16(v.x);
+    r.v[1] = f32_to_bf16(v.y);
+    r.v[2] = f32_to_bf16(v.z);
+    r.v[3] = f32_to_bf16(v.w);
+    *(ushort4x*)p = r;
+  }
+};
+
 // ---------------------------------------------------------------------------
 // embedding
 // ---------------------------------------------------------------------------
@@ -139,8 +164,8 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
     int C, int taps, int silu) {
-  const int t = blockIdx.y;
-  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int s = row_seq[t];
   const int r0 = seq_cu[s];
@@ -202,8 +227,8 @@ __global__ __launch_bounds__(256) void causal_conv_vec8_kernel(
     const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
     int C, int taps, int silu) {
-  const int t = blockIdx.y;
-  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (c >= C) return;
   const int s = row_seq[t];
   const int r0 = seq_cu[s];
@@ -243,8 +268,8 @@ __global__ __launch_bounds__(256) void causal_conv_tile_kernel(
     const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
     int Trows, int C, int silu) {
-  const int t0 = blockIdx.y * ROWS;
-  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const int t0 = blockIdx.x * ROWS;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (c >= C) return;
   float wr[8][TAPS];
 #pragma unroll
@@ -288,7 +313,7 @@ __global__ __launch_bounds__(256) void causal_conv_tile_kernel(
     }
     if (silu) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = silu_f32(acc[e]);
+      for (int e = 0; e < 8; ++e) acc[e] *= sigmoid_for<T>(acc[e]);
     }
     Row8<T>::st(out + (int64_t)t * C + c, acc);
   }
@@ -362,7 +387,7 @@ void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
 #define LAUNCH_CONV_TILE(TP)                                                  \
   hipLaunchKernelGGL(                                                        \
       (causal_conv_tile_kernel<act_t, TP, 4>),                               \
-      dim3((C / 8 + 255) / 256, (T + 3) / 4), dim3(256), 0, stream,          \
+      dim3((T + 3) / 4, (C / 8 + 255) / 256), dim3(256), 0, stream,          \
       (act_t*)out.data_ptr(), (const act_t*)x.data_ptr(),                    \
       (int64_t)x.stride(0), (const float*)w.data_ptr(),                      \
       bias.has_value() ? (const float*)bias->data_ptr() : nullptr,           \
@@ -376,7 +401,7 @@ void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
     else if (vec8 && taps == 2) LAUNCH_CONV_TILE(2);
     else if (vec8)
       hipLaunchKernelGGL(
-          (causal_conv_vec8_kernel<act_t>), dim3((C / 8 + 255) / 256, T),
+          (causal_conv_vec8_kernel<act_t>), dim3(T, (C / 8 + 255) / 256),
           dim3(256), 0, stream, (act_t*)out.data_ptr(),
           (const act_t*)x.data_ptr(), (int64_t)x.stride(0),
           (const float*)w.data_ptr(),
@@ -387,7 +412,7 @@ void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
           (const int32_t*)row_seq.data_ptr(), C, taps, silu ? 1 : 0);
     else
     hipLaunchKernelGGL(
-        (causal_conv_kernel<act_t>), dim3((C + 255) / 256, T), dim3(256), 0,
+        (causal_conv_kernel<act_t>), dim3(T, (C + 255) / 256), dim3(256), 0,
         stream, (act_t*)out.data_ptr(), (const act_t*)x.data_ptr(),
         (int64_t)x.stride(0), (const float*)w.data_ptr(),
         bias.has_value() ? (const float*)bias->data_ptr() : nullptr,
@@ -417,8 +442,8 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(
     const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
     int Trows, int D, int M) {
-  const int t = blockIdx.y;
-  const int d = blockIdx.x * 256 + threadIdx.x;
+  const int t = blockIdx.x;
+  const int d = blockIdx.y * 256 + threadIdx.x;
   if (d >= D) return;
   const int s = row_seq[t];
   const int r0 = seq_cu[s];
@@ -437,6 +462,44 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(
   for (int m = 0; m < M; ++m)
     Act<T>::st(out + ((int64_t)m * Trows + t) * D + d,
                cur + diff * mu[m * D + d]);
+}
+
+// D % 8 == 0: one thread per (row, 8 channels), 16-byte accesses
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_mix_vec8_kernel(
+    T* __restrict__ out, const T* __restrict__ h, const float* __restrict__ mu,
+    float* __restrict__ state, const int32_t* __restrict__ seq_cu,
+    const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ row_seq,
+    int Trows, int D, int M) {
+  const int t = blockIdx.x;
+  const int d = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (d >= D) return;
+  const int s = row_seq[t];
+  const int r0 = seq_cu[s];
+  float cur[8], prev[8];
+  Row8<T>::ld(h + (int64_t)t * D + d, cur);
+  if (t > r0) {
+    Row8<T>::ld(h + (int64_t)(t - 1) * D + d, prev);
+  } else {
+    float* st = state + (int64_t)seq_slots[s] * D + d;
+    if (seq_start[s] > 0) {
+      Row8<float>::ld(st, prev);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) prev[e] = 0.0f;
+    }
+    float last[8];
+    Row8<T>::ld(h + (int64_t)(seq_cu[s + 1] - 1) * D + d, last);
+    Row8<float>::st(st, last);
+  }
+  for (int m = 0; m < M; ++m) {
+    float w[8], y[8];
+    Row8<float>::ld(mu + (int64_t)m * D + d, w);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = cur[e] + (prev[e] - cur[e]) * w[e];
+    Row8<T>::st(out + ((int64_t)m * Trows + t) * D + d, y);
+  }
 }
 
 void token_shift_mix(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
@@ -458,8 +521,18 @@ void token_shift_mix(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
   IGW_DISPATCH_ACT(h, {
+    if (D % 8 == 0)
+      hipLaunchKernelGGL(
+          (token_shift_mix_vec8_kernel<act_t>), dim3(T, (D / 8 + 255) / 256),
+          dim3(256), 0, stream, (act_t*)out.data_ptr(),
+          (const act_t*)h.data_ptr(), (const float*)mu.data_ptr(),
+          (float*)state.data_ptr(), (const int32_t*)seq_cu.data_ptr(),
+          (const int32_t*)seq_start.data_ptr(),
+          (const int32_t*)seq_slots.data_ptr(),
+          (const int32_t*)row_seq.data_ptr(), T, D, M);
+    else
     hipLaunchKernelGGL(
-        (token_shift_mix_kernel<act_t>), dim3((D + 255) / 256, T), dim3(256),
+        (token_shift_mix_kernel<act_t>), dim3(T, (D + 255) / 256), dim3(256),
         0, stream, (act_t*)out.data_ptr(), (const act_t*)h.data_ptr(),
         (const float*)mu.data_ptr(), (float*)state.data_ptr(),
         (const int32_t*)seq_cu.data_ptr(), (const int32_t*)seq_start.data_ptr(),
@@ -581,88 +654,129 @@ void ssm_gates(torch::Tensor out, torch::Tensor dt_pre, torch::Tensor a_log) {
 }
 
 // ---------------------------------------------------------------------------
-// read-out epilogue: a wave takes HNG_PAIRS consecutive (row, norm group)
-// pairs at once (all their loads are in flight together; the values wait
-// in registers between the statistic and the store), four waves per
-// workgroup.  VPL = values per lane: group <= 64 * VPL.
+// read-out epilogue over o fp32 [T, C], C = H * P: optional division of
+// every head by max(|den|, floor) + 1e-6 (den, floor [T, H]), RMS norm in
+// groups of `group` channels times w, sigmoid / silu gate before or after.
+// A wave takes HNG_PAIRS consecutive (row, group) pairs at once (all their
+// loads are in flight together; the values wait in registers between the
+// statistic and the store), four waves per workgroup; a lane holds VPL
+// runs of VW consecutive channels (16-byte loads when VW = 4):
+// group <= 64 * VPL * VW.
 // ---------------------------------------------------------------------------
 constexpr int HNG_PAIRS = 4;
 
-template <typename T, int VPL>
+template <typename T, int VW>
+DEVINLINE void hng_load(const float* o, const T* g, float* v, float* z) {
+  if constexpr (VW == 4) {
+    const float4 a = *(const float4*)o;
+    const float4 b = Val4<T>::ld(g);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    z[0] = b.x; z[1] = b.y; z[2] = b.z; z[3] = b.w;
+  } else if constexpr (VW == 2) {
+    const float2 a = *(const float2*)o;
+    v[0] = a.x; v[1] = a.y;
+    z[0] = Act<T>::ld(g);
+    z[1] = Act<T>::ld(g + 1);
+  } else {
+    v[0] = *o;
+    z[0] = Act<T>::ld(g);
+  }
+}
+
+// gate value in the activation type's precision class: exact functions
+// for fp32 activations, the hardware exp / rcp for bf16
+template <typename T>
+DEVINLINE float gate_value(float z, int silu) {
+  const float s = sigmoid_for<T>(z);
+  return silu ? z * s : s;
+}
+
+template <typename T, int VPL, int VW>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(
     T* __restrict__ out, const float* __restrict__ o,
     const T* __restrict__ gate, int64_t gate_stride,
-    const float* __restrict__ w, const float* __restrict__ floor_, int H,
-    int P, int PP, int group, float eps, int gate_silu, int gate_first,
-    int64_t npairs) {
+    const float* __restrict__ w, const float* __restrict__ den,
+    const float* __restrict__ floor_, int H, int P, int group, float eps,
+    int gate_silu, int gate_first, int64_t npairs) {
   const int lane = threadIdx.x & 63;
   const int C = H * P;
   const int ng = C / group;
-  const int64_t first =
-      ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * HNG_PAIRS;
-  // where channel c0 + i sits in o, without a division per element when
-  // the rows are dense (PP == P) or the group is one head
-  const bool dense = PP == P;
+  // pairs are numbered row-major (row, group); npairs < 2^31 (host check)
+  const int first = (blockIdx.x * 4 + (threadIdx.x >> 6)) * HNG_PAIRS;
+  const int np = (int)npairs;
+  const int t0 = first / ng, g0 = first - t0 * ng;
   const bool one_head = group == P;
-  float val[HNG_PAIRS][VPL], gz[HNG_PAIRS][VPL], inv_den[HNG_PAIRS];
+  int tj[HNG_PAIRS], gj[HNG_PAIRS];
 #pragma unroll
   for (int j = 0; j < HNG_PAIRS; ++j) {
-    const int64_t pair = min(first + j, npairs - 1);
-    const int t = (int)(pair / ng), g = (int)(pair % ng);
-    const int c0 = g * group;
-    const float* orow = o + (int64_t)t * H * PP;
-    const T* grow = gate + (int64_t)t * gate_stride;
-    inv_den[j] = 1.0f;
-    if (floor_ != nullptr && one_head)
-      inv_den[j] = 1.0f / (fmaxf(fabsf(orow[g * PP + P]),
-                                 floor_[(int64_t)t * H + g]) + 1e-6f);
+    // HNG_PAIRS <= ng or not: walk (row, group) forward, clamp at the end
+    int g = g0 + j, t = t0;
+    while (g >= ng) { g -= ng; ++t; }
+    if (first + j >= np) { t = (np - 1) / ng; g = (np - 1) - t * ng; }
+    tj[j] = t;
+    gj[j] = g;
+  }
+  float val[HNG_PAIRS][VPL][VW], gz[HNG_PAIRS][VPL][VW];
+  float scl[HNG_PAIRS][VPL];
+#pragma unroll
+  for (int j = 0; j < HNG_PAIRS; ++j) {
+    const int t = tj[j], c0 = gj[j] * group;
 #pragma unroll
     for (int e = 0; e < VPL; ++e) {
-      const int i = lane + 64 * e;
-      float v = 0.0f, z = 0.0f;
+      const int i = (lane + 64 * e) * VW;
+      scl[j][e] = 1.0f;
+#pragma unroll
+      for (int x = 0; x < VW; ++x) val[j][e][x] = gz[j][e][x] = 0.0f;
       if (i < group) {
         const int c = c0 + i;
-        if (dense) {
-          v = orow[c];
-        } else if (one_head) {
-          v = orow[g * PP + i];
-        } else {
-          const int h = c / P, p = c % P;
-          v = orow[h * PP + p];
-          if (floor_ != nullptr)
-            v = v / (fmaxf(fabsf(orow[h * PP + P]),
-                           floor_[(int64_t)t * H + h]) + 1e-6f);
+        hng_load<T, VW>(o + (int64_t)t * C + c,
+                        gate + (int64_t)t * gate_stride + c, val[j][e],
+                        gz[j][e]);
+        if (den != nullptr) {
+          // VW channels never straddle a head: P % VW == 0
+          const int h = one_head ? gj[j] : c / P;
+          const float d = fabsf(den[(int64_t)t * H + h]);
+          const float f = floor_ ? floor_[(int64_t)t * H + h] : 0.0f;
+          scl[j][e] = 1.0f / (fmaxf(d, f) + 1e-6f);
         }
-        z = Act<T>::ld(grow + c);
       }
-      val[j][e] = v;
-      gz[j][e] = z;
     }
   }
 #pragma unroll
   for (int j = 0; j < HNG_PAIRS; ++j) {
     float sq = 0.0f;
 #pragma unroll
-    for (int e = 0; e < VPL; ++e) {
-      const float z = gz[j][e];
-      const float a = gate_silu ? silu_f32(z) : 1.0f / (1.0f + expf(-z));
-      float v = val[j][e] * inv_den[j];
-      if (gate_first) v *= a;
-      gz[j][e] = a;
-      val[j][e] = v;
-      if (lane + 64 * e < group) sq += v * v;
-    }
+    for (int e = 0; e < VPL; ++e)
+#pragma unroll
+      for (int x = 0; x < VW; ++x) {
+        const float z = gz[j][e][x];
+        const float a = gate_value<T>(z, gate_silu);
+        float v = val[j][e][x] * scl[j][e];
+        if (gate_first) v *= a;
+        gz[j][e][x] = a;
+        val[j][e][x] = v;
+        sq += v * v;        // entries past the group are zero
+      }
     const float rstd = 1.0f / sqrtf(wave_reduce_sum(sq) / (float)group + eps);
-    const int64_t pair = first + j;
-    if (pair >= npairs) continue;
-    const int t = (int)(pair / ng), c0 = (int)(pair % ng) * group;
+    if (first + j >= np) continue;
+    const int t = tj[j], c0 = gj[j] * group;
 #pragma unroll
     for (int e = 0; e < VPL; ++e) {
-      const int i = lane + 64 * e;
+      const int i = (lane + 64 * e) * VW;
       if (i >= group) continue;
-      float v = val[j][e] * rstd * w[c0 + i];
-      if (!gate_first) v *= gz[j][e];
-      Act<T>::st(out + (int64_t)t * C + c0 + i, v);
+      float r[VW];
+#pragma unroll
+      for (int x = 0; x < VW; ++x) {
+        r[x] = val[j][e][x] * rstd * w[c0 + i + x];
+        if (!gate_first) r[x] *= gz[j][e][x];
+      }
+      T* dst = out + (int64_t)t * C + c0 + i;
+      if constexpr (VW == 4) {
+        Val4<T>::st(dst, make_float4(r[0], r[1], r[2], r[3]));
+      } else {
+#pragma unroll
+        for (int x = 0; x < VW; ++x) Act<T>::st(dst + x, r[x]);
+      }
     }
   }
 }
@@ -672,9 +786,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(
     T* __restrict__ out, const float* __restrict__ o,
     const T* __restrict__ gate, int64_t gate_stride,
-    const float* __restrict__ w, const float* __restrict__ floor_, int H,
-    int P, int PP, int group, float eps, int gate_silu, int gate_first,
-    int64_t npairs) {
+    const float* __restrict__ w, const float* __restrict__ den,
+    const float* __restrict__ floor_, int H, int P, int group, float eps,
+    int gate_silu, int gate_first, int64_t npairs) {
   const int lane = threadIdx.x & 63;
   const int C = H * P;
   const int ng = C / group;
@@ -682,16 +796,16 @@ __global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(
   if (pair >= npairs) return;
   const int t = (int)(pair / ng), g = (int)(pair % ng);
   const int c0 = g * group;
-  const float* orow = o + (int64_t)t * H * PP;
+  const float* orow = o + (int64_t)t * C;
   const T* grow = gate + (int64_t)t * gate_stride;
   auto value = [&](int i) {
     const int c = c0 + i;
-    if (PP == P) return orow[c];
-    const int h = c / P, p = c % P;
-    float v = orow[h * PP + p];
-    if (floor_ != nullptr)
-      v = v / (fmaxf(fabsf(orow[h * PP + P]), floor_[(int64_t)t * H + h]) +
-               1e-6f);
+    float v = orow[c];
+    if (den != nullptr) {
+      const int h = c / P;
+      const float f = floor_ ? floor_[(int64_t)t * H + h] : 0.0f;
+      v = v / (fmaxf(fabsf(den[(int64_t)t * H + h]), f) + 1e-6f);
+    }
     return v;
   };
   float sq = 0.0f;
@@ -719,11 +833,11 @@ __global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(
 void head_norm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
                     torch::Tensor w, double eps, int64_t group,
                     int64_t gate_act, bool gate_first,
+                    c10::optional<torch::Tensor> den,
                     c10::optional<torch::Tensor> floor_) {
   TORCH_CHECK(o.is_cuda() && o.dtype() == torch::kFloat32 &&
               o.is_contiguous() && o.dim() == 3);
-  const int T = o.size(0), H = o.size(1), PP = o.size(2);
-  const int P = floor_.has_value() ? PP - 1 : PP;
+  const int T = o.size(0), H = o.size(1), P = o.size(2);
   const int C = H * P;
   TORCH_CHECK(P >= 1 && group >= 1 && C % group == 0,
               "norm groups must divide the channels");
@@ -732,28 +846,42 @@ void head_norm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor gate,
               gate.size(1) == C && gate.dtype() == out.dtype());
   TORCH_CHECK(w.dtype() == torch::kFloat32 && w.numel() == C &&
               w.is_contiguous());
-  if (floor_.has_value())
-    TORCH_CHECK(floor_->dtype() == torch::kFloat32 &&
-                floor_->is_contiguous() && floor_->numel() == (int64_t)T * H);
+  TORCH_CHECK(den.has_value() || !floor_.has_value(),
+              "a floor needs the normaliser it bounds");
+  for (const auto* x : {&den, &floor_})
+    if (x->has_value())
+      TORCH_CHECK((*x)->dtype() == torch::kFloat32 && (*x)->is_contiguous() &&
+                  (*x)->numel() == (int64_t)T * H);
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
   const int64_t npairs = (int64_t)T * (C / group);
+  TORCH_CHECK(npairs < (int64_t)1 << 31, "too many (row, group) pairs");
+  const int64_t ge = gate.element_size();
+  const bool vec4 = P % 4 == 0 && group % 4 == 0 &&
+                    (gate.stride(0) * ge) % (4 * ge) == 0 &&
+                    reinterpret_cast<uintptr_t>(gate.data_ptr()) % (4 * ge) ==
+                        0;
 #define HNG_ARGS                                                              \
   (act_t*)out.data_ptr(), (const float*)o.data_ptr(),                         \
       (const act_t*)gate.data_ptr(), (int64_t)gate.stride(0),                 \
       (const float*)w.data_ptr(),                                             \
+      den.has_value() ? (const float*)den->data_ptr() : nullptr,              \
       floor_.has_value() ? (const float*)floor_->data_ptr() : nullptr, H, P,  \
-      PP, (int)group, (float)eps, gate_act == 1 ? 1 : 0, gate_first ? 1 : 0,  \
+      (int)group, (float)eps, gate_act == 1 ? 1 : 0, gate_first ? 1 : 0,      \
       npairs
-#define LAUNCH_HNG(VPL)                                                       \
-  hipLaunchKernelGGL((head_norm_gate_kernel<act_t, VPL>),                     \
+#define LAUNCH_HNG(VPL, VW)                                                   \
+  hipLaunchKernelGGL((head_norm_gate_kernel<act_t, VPL, VW>),                 \
                      dim3((npairs + 4 * HNG_PAIRS - 1) / (4 * HNG_PAIRS)),    \
                      dim3(256), 0, stream, HNG_ARGS)
   IGW_DISPATCH_ACT(out, {
-    if (group <= 64) LAUNCH_HNG(1);
-    else if (group <= 128) LAUNCH_HNG(2);
-    else if (group <= 256) LAUNCH_HNG(4);
-    else if (group <= 512) LAUNCH_HNG(8);
+    if (vec4 && group <= 64) LAUNCH_HNG(1, 1);
+    else if (vec4 && group <= 128) LAUNCH_HNG(1, 2);
+    else if (vec4 && group <= 256) LAUNCH_HNG(1, 4);
+    else if (vec4 && group <= 512) LAUNCH_HNG(2, 4);
+    else if (vec4 && group <= 1024) LAUNCH_HNG(4, 4);
+    else if (group <= 64) LAUNCH_HNG(1, 1);
+    else if (group <= 128) LAUNCH_HNG(2, 1);
+    else if (group <= 256) LAUNCH_HNG(4, 1);
     else
       hipLaunchKernelGGL((head_norm_gate_wide_kernel<act_t>),
                          dim3((npairs + 3) / 4), dim3(256), 0, stream,
@@ -863,17 +991,44 @@ __global__ __launch_bounds__(RROW_BLOCK) void rmsnorm_pair_mean_kernel(
   const T* ar = a + row * D;
   const T* br = b + row * D;
   float sa = 0.0f, sb = 0.0f;
-  for (int d = threadIdx.x; d < D; d += RROW_BLOCK) {
-    const float x = Act<T>::ld(ar + d), y = Act<T>::ld(br + d);
-    sa += x * x;
-    sb += y * y;
+  if (D % 8 == 0) {
+    for (int d = threadIdx.x * 8; d < D; d += RROW_BLOCK * 8) {
+      float x[8], y[8];
+      Row8<T>::ld(ar + d, x);
+      Row8<T>::ld(br + d, y);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        sa += x[e] * x[e];
+        sb += y[e] * y[e];
+      }
+    }
+  } else {
+    for (int d = threadIdx.x; d < D; d += RROW_BLOCK) {
+      const float x = Act<T>::ld(ar + d), y = Act<T>::ld(br + d);
+      sa += x * x;
+      sb += y * y;
+    }
   }
   const float ra = 1.0f / sqrtf(rrow_block_sum(sa, lds) / (float)D + eps);
   const float rb = 1.0f / sqrtf(rrow_block_sum(sb, lds) / (float)D + eps);
-  for (int d = threadIdx.x; d < D; d += RROW_BLOCK)
-    Act<T>::st(out + row * D + d,
-               0.5f * (Act<T>::ld(ar + d) * ra * wa[d] +
-                       Act<T>::ld(br + d) * rb * wb[d]));
+  if (D % 8 == 0) {
+    for (int d = threadIdx.x * 8; d < D; d += RROW_BLOCK * 8) {
+      float x[8], y[8], u[8], v[8], r[8];
+      Row8<T>::ld(ar + d, x);
+      Row8<T>::ld(br + d, y);
+      Row8<float>::ld(wa + d, u);
+      Row8<float>::ld(wb + d, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        r[e] = 0.5f * (x[e] * ra * u[e] + y[e] * rb * v[e]);
+      Row8<T>::st(out + row * D + d, r);
+    }
+  } else {
+    for (int d = threadIdx.x; d < D; d += RROW_BLOCK)
+      Act<T>::st(out + row * D + d,
+                 0.5f * (Act<T>::ld(ar + d) * ra * wa[d] +
+                         Act<T>::ld(br + d) * rb * wb[d]));
+  }
 }
 
 void rmsnorm_pair_mean(torch::Tensor out, torch::Tensor a, torch::Tensor b,

@@ -146,6 +146,7 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
       window > 0 ? max(0, P0 + qoff - window + 1) / BN * BN : 0;
 
   // the next K/V tile travels in registers while the current one is used
+  // (a second tile in flight costs more in occupancy than it hides)
   constexpr int KIT = BN * NP / 8 / 256, VIT = BN * PP / 8 / 256;
   ushort8 kreg[KIT], vreg[VIT];
   auto fetch = [&](int kbase) {
@@ -206,6 +207,8 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
     }
     __syncthreads();
     if (kbase + BN < kend) fetch(kbase + BN);
+    // a wave none of whose 16 rows exists only helps with the staging
+    if (wave * 16 >= nrows) continue;
 
     float4v acc_s[4];
 #pragma unroll

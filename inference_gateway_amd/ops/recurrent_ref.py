@@ -129,7 +129,8 @@ def outer_scan_ref(q, k, v, decay, kscale, bonus, skip, state, seq_cu,
       bonus u:     o_t = (S + diag(u) k_t v_t^T)^T q_t   (reads the old)
       o_t = o_t * qscale + skip_h * v_t
     q, k [T, G, N] (head h uses group h // (H/G)), v [T, H, P], decay
-    [T, H, Nd] with Nd in {1, N}; returns fp32 [T, H, PP]."""
+    [T, H, Nd] with Nd in {1, N}; returns fp32 (o [T, H, P], read-out of
+    the ones column [T, H] or None)."""
     T, H, P = v.shape
     G, N = q.shape[1], q.shape[2]
     PP = P + (1 if ones_col else 0)
@@ -165,20 +166,23 @@ def outer_scan_ref(q, k, v, decay, kscale, bonus, skip, state, seq_cu,
     out = out * qscale
     if skip is not None:
         out[:, :, :P] += skip[None, :, None] * v.float()
-    return out
+    if ones_col:
+        return out[:, :, :P].contiguous(), out[:, :, P].contiguous()
+    return out, None
 
 
-def head_norm_gate_ref(o, gate, w, eps, group, gate_act, gate_first, floor,
-                       out_dtype):
-    """o fp32 [T, H, PP].  With floor [T, H] the last column of o is a
-    normaliser: o <- o[..., :P] / (max(|o[..., P]|, floor) + 1e-6).
-    Then, over the flattened channels C = H*P: gate (sigmoid or silu of
-    the pre-activations `gate` [T, C]) before or after an RMS norm in
-    groups of `group` channels, times w."""
-    T, H, PP = o.shape
-    if floor is not None:
-        den = torch.maximum(o[:, :, PP - 1].abs(), floor) + 1e-6
-        o = o[:, :, :PP - 1] / den[:, :, None]
+def head_norm_gate_ref(o, gate, w, eps, group, gate_act, gate_first, den,
+                       floor, out_dtype):
+    """o fp32 [T, H, P].  With den [T, H]: o <- o / (max(|den|, floor) +
+    1e-6) per head (floor None = 0).  Then, over the flattened channels
+    C = H*P: gate (sigmoid or silu of the pre-activations `gate` [T, C])
+    before or after an RMS norm in groups of `group` channels, times w."""
+    T, H, P = o.shape
+    if den is not None:
+        d = den.abs()
+        if floor is not None:
+            d = torch.maximum(d, floor)
+        o = o / (d + 1e-6)[:, :, None]
     y = o.reshape(T, -1)
     C = y.shape[1]
     g = gate.float()

@@ -312,14 +312,20 @@ def test_outer_scan_forms(device, shape):
         cu, st, so, rs, _ = ragged(rows, starts, sl, device)
         cat = [torch.cat([p[i] for p in parts]).to(device)
                if parts[0][i] is not None else None for i in range(6)]
-        out = ops.outer_scan(
+        out, nrm = ops.outer_scan(
             cat[0], cat[1], cat[2], cat[5].contiguous(), cat[4],
             None if u is None else u.to(device),
             None if skip is None else skip.to(device), state, cu, st, so,
             rows, ops.DECAY_EXP_NEG_EXP if form == "decay"
             else ops.DECAY_LINEAR, ones, qscale)
-        np.testing.assert_allclose(out.cpu().numpy(), np.concatenate(want),
+        want = np.concatenate(want)
+        np.testing.assert_allclose(out.cpu().numpy(), want[:, :, :P],
                                    atol=2e-4, rtol=2e-4)
+        if ones:
+            np.testing.assert_allclose(nrm.cpu().numpy(), want[:, :, P],
+                                       atol=2e-4, rtol=2e-4)
+        else:
+            assert nrm is None
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -368,8 +374,10 @@ def test_head_norm_gate_modes(device):
     den = np.maximum(np.abs(od[:, :, P]), fd) + 1e-6
     ref = oracle.rms_unit(od[:, :, :P] / den[:, :, None], 1e-5).reshape(
         T, -1) * w.double().numpy() * oracle.sigmoid(gd)
-    got = ops.head_norm_gate(o.to(device), gate[:, :H * P].to(device),
-                             w.to(device), 1e-5, P, ops.GATE_SIGMOID, False,
+    got = ops.head_norm_gate(o[:, :, :P].contiguous().to(device),
+                             gate[:, :H * P].to(device), w.to(device), 1e-5,
+                             P, ops.GATE_SIGMOID, False,
+                             o[:, :, P].contiguous().to(device),
                              floor.to(device), torch.float32)
     np.testing.assert_allclose(got.cpu().numpy(), ref, atol=2e-5, rtol=2e-5)
     # silu gate first, norm in two parts that span heads
@@ -379,13 +387,14 @@ def test_head_norm_gate_modes(device):
         * w.double().numpy()
     got = ops.head_norm_gate(o2.to(device), gate[:, :H * P].to(device),
                              w.to(device), 1e-5, H * P // 2, ops.GATE_SILU,
-                             True, None, torch.float32)
+                             True, None, None, torch.float32)
     np.testing.assert_allclose(got.cpu().numpy(), ref, atol=2e-5, rtol=2e-5)
 
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dims", [(3, 5, 130, 650), (2, 4, 96, 384),
-                                  (4, 3, 70, 70)])
+                                  (4, 3, 70, 70), (3, 2, 128, 128),
+                                  (2, 8, 128, 1024), (2, 9, 128, 1152)])
 def test_head_norm_gate_group_sizes(device, dims):
     """Groups from one head to several, up to the two-pass kernel."""
     T, H, P, group = dims
@@ -404,7 +413,7 @@ def test_head_norm_gate_group_sizes(device, dims):
             y = y * a
         got = ops.head_norm_gate(o.to(device), gate.to(device),
                                  w.to(device), 1e-6, group, ops.GATE_SILU,
-                                 first, None, torch.float32)
+                                 first, None, None, torch.float32)
         np.testing.assert_allclose(got.cpu().numpy(), y, atol=3e-5,
                                    rtol=3e-5)
 
@@ -681,6 +690,60 @@ def test_greedy_generation_through_scheduler(tmp_path, device, mode):
         eng.step()
     for rid, p in zip(rids, prompts):
         assert eng.get_output(rid).token_ids == _greedy(cfg, W, p, 6)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_preemption_restarts_every_state(tmp_path, device):
+    """A pool too small for both requests: the newer one is preempted,
+    its slot buffers dropped with its pages, and it resumes by re-running
+    its folded prompt from position 0."""
+    cfg = cfg_small()
+    W = oracle.random_weights(cfg, 26)
+    prompts = [toks(7, cfg["vocab"], 41), toks(6, cfg["vocab"], 42)]
+    refs = [_greedy(cfg, W, p, 10) for p in prompts]
+    eng = make_engine(tmp_path, cfg, W, device, blocks=8, block=4)
+    sp = SamplingParams(max_new_tokens=10, temperature=0.0)
+    ids = [eng.add_request(p, sp) for p in prompts]
+    for _ in range(300):
+        if eng.is_finished():
+            break
+        eng.step()
+    assert eng.scheduler.num_preemptions > 0
+    for i, r in zip(ids, refs):
+        assert eng.get_output(i).token_ids == r
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_forked_group_copies_every_slot_buffer(tmp_path, device):
+    """n=2 from one prefill: the branch shares the prompt's pages and
+    starts from a COPY of the parent's memories, filter histories,
+    previous row and previous token."""
+    cfg = cfg_small()
+    W = oracle.random_weights(cfg, 27)
+    prompt = toks(10, cfg["vocab"], 43)     # 2 full pages + a partial one
+    ref = _greedy(cfg, W, prompt, 5)
+    eng = make_engine(tmp_path, cfg, W, device, blocks=32)
+    ids = eng.add_request_group(
+        prompt, SamplingParams(max_new_tokens=5, temperature=0.0), n=2)
+    while not eng.is_finished():
+        eng.step()
+    assert eng.num_forks == 1
+    for i in ids:
+        assert eng.get_output(i).token_ids == ref
+
+
+def test_table_sizes_from_tensors(tmp_path):
+    """A config.json that leaves out the table sizes takes them from
+    the checkpoint header."""
+    cfg = cfg_ones()
+    W = oracle.random_weights(cfg, 28)
+    lean = {k: v for k, v in cfg.items() if k != "max_positions"}
+    lean["embedding"] = {"scale": cfg["embedding"]["scale"],
+                         "bigram": {"mul_prev": 1, "mul_cur": 1}}
+    path = oracle.save_checkpoint(tmp_path / "m", lean, W)
+    mc = model_config_from_dir(path)
+    assert mc.max_position == cfg["max_positions"]
+    assert mc.pair_hash.buckets == cfg["embedding"]["bigram"]["buckets"]
 
 
 def test_registry_config_and_loader_errors(tmp_path):

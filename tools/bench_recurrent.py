@@ -193,15 +193,16 @@ def _kernels(sz):
         ms = torch.zeros(nseq, H, device=dev)
         t = _time(lambda: ops.mlstm_gates(pre, 15.0, ms, cu, st, sl), it)
         out[f"mlstm_gates_{tag}"] = _entry(t, bytes_=T * H * 20.0)
-        o = torch.randn(T, H, P + 1, device=dev)
+        o = torch.randn(T, H, P, device=dev)
+        dn = torch.randn(T, H, device=dev)
         gate = torch.randn(T, H * P, device=dev, dtype=bf)
         w = torch.ones(H * P, device=dev)
         fl = torch.rand(T, H, device=dev)
         t = _time(lambda: ops.head_norm_gate(o, gate, w, 1e-6, P,
-                                             ops.GATE_SIGMOID, False, fl,
-                                             bf), it)
+                                             ops.GATE_SIGMOID, False, dn,
+                                             fl, bf), it)
         out[f"head_norm_gate_{tag}"] = _entry(
-            t, bytes_=T * H * ((P + 1) * 4.0 + P * 4.0))
+            t, bytes_=T * H * (P * 4.0 + 8 + P * 4.0))
 
     # ---- row kernels on 8192 rows (8 sequences of 1024) ----
     T, cu, st, sl, row_seq = seqs(8, 1024, 0)
