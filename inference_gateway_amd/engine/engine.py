@@ -142,6 +142,11 @@ class LLMEngine:
         # sequence-level batch metadata (row -> sequence maps, state
         # slots) is only assembled for models that read it
         self._seq_meta = getattr(self.model, "needs_seq_meta", False)
+        # a model with a learned position table serves no sequence longer
+        # than the table
+        rows = getattr(self.model, "position_table_rows", None)
+        if rows and cfg.max_model_len > rows:
+            cfg.max_model_len = int(rows)
         if is_recurrent(cfg.model) and cfg.enable_prefix_caching:
             raise ValueError(
                 "prefix caching cannot serve a model with recurrent "

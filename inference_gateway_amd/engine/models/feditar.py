@@ -359,6 +359,8 @@ class FeditarForCausalLM(nn.Module):
             for i in range(cfg.num_layers))
         self.final_norm_w = _one_plus(D, device, "final.norm")
         self.tap = None    # debugging hook: called with (layer, residual)
+        # the engine caps its sequence length at the learned table
+        self.position_table_rows = cfg.max_position
 
     def cache_specs(self) -> List[tuple]:
         """One entry per layer (a group of slot buffers, plus paged K/V

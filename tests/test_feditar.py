@@ -789,6 +789,41 @@ def test_preset_runs_and_forks_copy_state(tmp_path):
     assert all(bool((t[2] == 3).all()) for t in leaves)
 
 
+def test_local_provider_serves_a_checkpoint_directory(tmp_path):
+    """The gateway's local provider with LOCAL_MODEL=hf picks the
+    architecture from the directory's config.json and generates through
+    the async engine with sampling."""
+    import asyncio
+
+    from inference_gateway_amd.config import LocalConfig
+    from inference_gateway_amd.providers.local import LocalProvider
+
+    cfg = oracle.make_config(48, 300, [
+        oracle.mlstm_layer(2, 8, 6),
+        oracle.parallel_layer(2, 1, 8, 10, 3, 0.2, 16, 0.35, 9.0, 3, 4,
+                              ff=32)], max_positions=160)
+    W = oracle.random_weights(cfg, 35)
+    path = oracle.save_checkpoint(tmp_path / "m", cfg, W)
+    lc = LocalConfig(enabled=True, model="hf", max_num_seqs=4,
+                     max_model_len=128)
+    lc.num_gpu_blocks = 64
+    lc.weights_path = path
+    provider = LocalProvider(lc, device="cpu")
+    try:
+        assert isinstance(provider.engine.engine.cfg.model, FeditarConfig)
+
+        async def go(temp):
+            return await provider.chat_completions({
+                "model": "local/hf",
+                "messages": [{"role": "user", "content": "hi"}],
+                "max_tokens": 3, "temperature": temp, "top_p": 0.9})
+
+        assert asyncio.run(go(0))["usage"]["completion_tokens"] == 3
+        assert asyncio.run(go(0.8))["usage"]["completion_tokens"] == 3
+    finally:
+        provider.engine.shutdown()
+
+
 def test_trace_command(tmp_path):
     """bin/trace_run end to end on a small checkpoint: portions, a
     decoded token, a step with nothing wanted, a second request that
