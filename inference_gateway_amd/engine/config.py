@@ -596,6 +596,294 @@ def feditar_preset(name: str, width: int, vocab: int, pattern: str,
         max_position=max_position)
 
 
+# ---------------------------------------------------------------------------
+# Bozolorn: a per-layer decoder with sandwich norms (an RMS norm before
+# AND after every sublayer), a small per-layer token embedding added after
+# the feed-forward, and mixture-of-experts feed-forwards whose sigmoid
+# router picks experts inside the best expert groups.  Mixers: softmax
+# attention without rotation, with a linear distance bias, restricted to
+# position chunks and gated at its output (a layer may borrow another
+# layer's keys and values); or a PARALLEL pair of rotated softmax attention
+# with a unit sink in its denominator beside a gated delta-rule memory.
+# ---------------------------------------------------------------------------
+@dataclass
+class YarnRotarySpec:
+    """Interleaved-pair rotary positions on the first `dims` entries of a
+    head with YaRN frequency interpolation: with where(t) = dims *
+    ln(original / (2 pi t)) / (2 ln base), lo = max(floor(where(fast)),
+    0), hi = min(ceil(where(slow)), dims - 1) and ramp_i = clamp((i - lo)
+    / max(hi - lo, 0.001), 0, 1), pair i turns by position * (f_i /
+    factor * ramp_i + f_i * (1 - ramp_i)), f_i = base**(-2i/dims); cos
+    and sin are multiplied by 0.1 ln(factor) + 1.  factor <= 0 or 1 with
+    no `original` means plain rotation."""
+    base: float = 10000.0
+    dims: int = 0
+    factor: float = 0.0        # 0 => no interpolation
+    original: float = 0.0
+    fast: float = 32.0
+    slow: float = 1.0
+
+    def frequencies(self):
+        """([dims/2] angular steps as python floats, cos/sin factor)."""
+        import math
+
+        f = [self.base ** (-2.0 * i / self.dims)
+             for i in range(self.dims // 2)]
+        if not self.factor:
+            return f, 1.0
+
+        def where(turns):
+            return self.dims * math.log(
+                self.original / (2.0 * math.pi * turns)) / (
+                    2.0 * math.log(self.base))
+
+        lo = max(math.floor(where(self.fast)), 0)
+        hi = min(math.ceil(where(self.slow)), self.dims - 1)
+        out = []
+        for i, fi in enumerate(f):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            out.append(fi / self.factor * ramp + fi * (1.0 - ramp))
+        return out, 0.1 * math.log(self.factor) + 1.0
+
+
+@dataclass
+class ChunkBiasAttentionSpec:
+    """Softmax attention without rotation: score = q.k * scale - slope_h
+    * (i - j) with slope_h = 2**(-8 (h + 1) / heads); position i sees j
+    <= i of its own chunk of `chunk` positions (0 = plain causal);
+    sigmoid output gate.  kv_from = index of the layer whose keys and
+    values this layer reads instead of projecting its own (-1 = own)."""
+    heads: int = 1
+    kv_heads: int = 1
+    dim: int = 64
+    vdim: int = 64
+    scale: float = 0.0         # 0 => dim ** -0.5
+    chunk: int = 0
+    kv_from: int = -1
+
+    def __post_init__(self):
+        if not self.scale:
+            self.scale = float(self.dim) ** -0.5
+
+
+@dataclass
+class SinkAttentionSpec:
+    """Causal softmax attention with projection biases, per-head RMS
+    norm of queries and keys, partial rotary positions, and one more
+    term of score 0 and no value in the softmax denominator."""
+    heads: int = 1
+    kv_heads: int = 1
+    dim: int = 64
+    vdim: int = 64
+    scale: float = 0.0         # 0 => dim ** -0.5
+    rot: YarnRotarySpec = None  # None => no rotation
+
+    def __post_init__(self):
+        if not self.scale:
+            self.scale = float(self.dim) ** -0.5
+
+
+@dataclass
+class DeltaRuleSpec:
+    """Gated delta-rule memory: `kv_heads` query/key heads of `dim`
+    entries shared by groups of the `heads` value heads of `vdim`
+    entries; q, k, v pass a causal convolution of `conv` taps and silu."""
+    heads: int = 1
+    kv_heads: int = 1
+    dim: int = 64
+    vdim: int = 64
+    conv: int = 4
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+
+@dataclass
+class SinkDeltaPairSpec:
+    left: SinkAttentionSpec = None
+    right: DeltaRuleSpec = None
+
+
+@dataclass
+class GroupRoutedSpec:
+    """Clamped gated experts chosen by a sigmoid router: choice score =
+    sigmoid(logit) + correction; the experts form `groups` equal groups
+    of neighbours, a group scores the sum of its two best choice scores,
+    only experts of the best `keep` groups can be chosen; the `top`
+    chosen experts are weighted by their plain sigmoid scores."""
+    experts: int = 1
+    top: int = 1
+    groups: int = 1
+    keep: int = 1
+    expert_ff: int = 0
+    limit: float = 7.0
+
+
+@dataclass
+class BozolornConfig:
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: list               # LayerSpec(type="attention"|"parallel")
+    norm_eps: float = 1e-6
+    embed_scale: float = 1.0
+    side_dim: int = 0          # per-layer token embedding width; 0 = none
+    max_position: int = 1 << 20     # angles are computed, not tabulated
+    architecture: str = "Bozolorn"
+
+    def __post_init__(self):
+        for i, l in enumerate(self.layers):
+            if l.type != "attention" or l.mixer.kv_from < 0:
+                continue
+            src = l.mixer.kv_from
+            if not (0 <= src < i) or self.layers[src].type != "attention" \
+                    or self.layers[src].mixer.kv_from >= 0:
+                raise ValueError(
+                    f"layer {i}: kv_from must name an earlier attention "
+                    "layer that projects its own keys and values")
+            o = self.layers[src].mixer
+            if (o.kv_heads, o.dim, o.vdim) != (
+                    l.mixer.kv_heads, l.mixer.dim, l.mixer.vdim):
+                raise ValueError(
+                    f"layer {i}: key/value sizes differ from layer {src}'s")
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(l.mlp is not None for l in self.layers)
+
+    def kv_bytes_per_token(self, itemsize: int = 2) -> int:
+        """Paged bytes per token: the attention layers that own keys and
+        values and the attention half of every parallel mixer; the
+        delta-rule memories are fixed per slot."""
+        n = 0
+        for l in self.layers:
+            a = l.mixer.left if l.type == "parallel" else l.mixer
+            if l.type == "parallel" or a.kv_from < 0:
+                n += a.kv_heads * (a.dim + a.vdim) * itemsize
+        return max(itemsize, n)
+
+    @staticmethod
+    def from_dict(cfg: dict, name: str = "bozolorn",
+                  shapes: Optional[dict] = None) -> "BozolornConfig":
+        """Parse the design's config.json (every size and constant is in
+        it; `shapes` is accepted for symmetry with the other designs)."""
+
+        def rotary(r):
+            if not r:
+                return None
+            sc = r.get("scaling") or {}
+            return YarnRotarySpec(
+                base=float(r["base"]), dims=int(r["dims"]),
+                factor=float(sc.get("factor") or 0.0),
+                original=float(sc.get("original") or 0.0),
+                fast=float(sc.get("fast", 32.0)),
+                slow=float(sc.get("slow", 1.0)))
+
+        def attention(m):
+            kv_from = m.get("kv_from")
+            return ChunkBiasAttentionSpec(
+                heads=int(m["heads"]),
+                kv_heads=int(m.get("kv_heads") or m["heads"]),
+                dim=int(m["dim"]), vdim=int(m.get("vdim") or m["dim"]),
+                scale=float(m.get("scale") or 0.0),
+                chunk=int((m.get("mask") or {}).get("size") or 0),
+                kv_from=-1 if kv_from is None else int(kv_from))
+
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m = l.get("mixer") or {}
+            t = l["type"]
+            if t == "attention":
+                mixer = attention(m)
+            elif t == "parallel":
+                a, b = m["left"], m["right"]
+                mixer = SinkDeltaPairSpec(
+                    left=SinkAttentionSpec(
+                        heads=int(a["heads"]),
+                        kv_heads=int(a.get("kv_heads") or a["heads"]),
+                        dim=int(a["dim"]),
+                        vdim=int(a.get("vdim") or a["dim"]),
+                        scale=float(a.get("scale") or 0.0),
+                        rot=rotary(a.get("rot"))),
+                    right=DeltaRuleSpec(
+                        heads=int(b["heads"]),
+                        kv_heads=int(b.get("kv_heads") or b["heads"]),
+                        dim=int(b["dim"]),
+                        vdim=int(b.get("vdim") or b["dim"]),
+                        conv=int(b.get("conv") or 1)))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer {t!r}")
+            f = l.get("mlp")
+            if f is None:
+                mlp = None
+            elif f["kind"] == "moe":
+                r = f["router"]
+                gr = r.get("groups") or {}
+                mlp = GroupRoutedSpec(
+                    experts=int(r["experts"]), top=int(r["top"]),
+                    groups=int(gr.get("count") or 1),
+                    keep=int(gr.get("keep") or gr.get("count") or 1),
+                    expert_ff=int(f["expert"]["ff"]),
+                    limit=float(f["expert"]["limit"]))
+                if mlp.experts % mlp.groups:
+                    raise ValueError(
+                        f"layer {i}: {mlp.experts} experts do not split "
+                        f"into {mlp.groups} equal groups")
+            else:
+                raise ValueError(f"layer {i}: unknown mlp {f['kind']!r}")
+            layers.append(LayerSpec(type=t, mixer=mixer, mlp=mlp))
+        return BozolornConfig(
+            name=name, hidden_size=int(cfg["width"]),
+            vocab_size=int(cfg["vocab"]), layers=layers,
+            norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-6)),
+            embed_scale=float((cfg.get("embedding") or {}).get("scale",
+                                                               1.0)),
+            side_dim=int((cfg.get("token_side") or {}).get("dim") or 0))
+
+
+def bozolorn_preset(name: str, width: int, vocab: int, pattern: str,
+                    heads: int, kv_heads: int, dim: int, vdim: int,
+                    chunk: int, rot_dims: int, d_heads: int,
+                    d_kv_heads: int, d_dim: int, d_vdim: int,
+                    experts: int, top: int, groups: int, keep: int,
+                    expert_ff: int, conv: int = 4, limit: float = 7.0,
+                    side_dim: int = 0, rot_base: float = 1000000.0,
+                    yarn_factor: float = 0.0,
+                    yarn_original: float = 0.0) -> BozolornConfig:
+    """Layer pattern string: one token per layer — mixer `a` (chunked
+    attention), `a<j>` (the same, reading layer j's keys and values) or
+    `p` (parallel sink attention + delta rule), then `m` (experts) or
+    `-` (no feed-forward); e.g. "pm am pm a1m p-"."""
+    layers = []
+    for tok in pattern.split():
+        if tok[0] == "a":
+            typ, mixer = "attention", ChunkBiasAttentionSpec(
+                heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim,
+                chunk=chunk, kv_from=int(tok[1:-1]) if tok[1:-1] else -1)
+        else:
+            typ, mixer = "parallel", SinkDeltaPairSpec(
+                left=SinkAttentionSpec(
+                    heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim,
+                    rot=YarnRotarySpec(base=rot_base, dims=rot_dims,
+                                       factor=yarn_factor,
+                                       original=yarn_original)
+                    if rot_dims else None),
+                right=DeltaRuleSpec(heads=d_heads, kv_heads=d_kv_heads,
+                                    dim=d_dim, vdim=d_vdim, conv=conv))
+        mlp = GroupRoutedSpec(experts=experts, top=top, groups=groups,
+                              keep=keep, expert_ff=expert_ff,
+                              limit=limit) if tok[-1] == "m" else None
+        layers.append(LayerSpec(type=typ, mixer=mixer, mlp=mlp))
+    return BozolornConfig(name=name, hidden_size=width, vocab_size=vocab,
+                          layers=layers, embed_scale=float(width) ** 0.5,
+                          side_dim=side_dim)
+
+
 # Architectures from the public model cards (random-init weights — no network).
 MODEL_PRESETS = {
     "llama-3-8b": ModelConfig(
@@ -754,6 +1042,21 @@ MODEL_PRESETS = {
         "feditar-4k", width=4096, vocab=32000, pattern="x- s- pd pd",
         heads=32, kv_heads=8, dim=128, vdim=128, state=128, groups=8,
         ff=14336, norm_groups=8, decay_rank=64),
+    # tiny Bozolorn for CPU tests / smoke: both mixers, a borrowed
+    # key/value layer, a layer without feed-forward
+    "tiny-bozolorn": bozolorn_preset(
+        "tiny-bozolorn", width=96, vocab=320, pattern="pm am p- a1m",
+        heads=4, kv_heads=2, dim=24, vdim=16, chunk=20, rot_dims=16,
+        d_heads=4, d_kv_heads=2, d_dim=16, d_vdim=24, experts=6, top=2,
+        groups=3, keep=2, expert_ff=40, conv=3, limit=1.5, side_dim=8,
+        yarn_factor=4.0, yarn_original=64.0),
+    # layer-shape benchmark point at Llama-3-8B's width
+    "bozolorn-4k": bozolorn_preset(
+        "bozolorn-4k", width=4096, vocab=32000, pattern="pm am pm a1m",
+        heads=32, kv_heads=8, dim=128, vdim=128, chunk=1024, rot_dims=64,
+        d_heads=32, d_kv_heads=8, d_dim=128, d_vdim=128, experts=8, top=2,
+        groups=4, keep=2, expert_ff=14336, side_dim=64,
+        yarn_factor=4.0, yarn_original=4096.0),
     "tiny-moe": ModelConfig(
         name="tiny-moe",
         hidden_size=512,
@@ -894,6 +1197,19 @@ class EngineConfig:
     def tiny_feditar(**kw) -> "EngineConfig":
         defaults = dict(
             model=MODEL_PRESETS["tiny-feditar"],
+            num_gpu_blocks=64,
+            max_num_seqs=8,
+            max_batched_tokens=2048,
+            max_model_len=512,
+            use_hip_graphs=False,
+        )
+        defaults.update(kw)
+        return EngineConfig(**defaults)
+
+    @staticmethod
+    def tiny_bozolorn(**kw) -> "EngineConfig":
+        defaults = dict(
+            model=MODEL_PRESETS["tiny-bozolorn"],
             num_gpu_blocks=64,
             max_num_seqs=8,
             max_batched_tokens=2048,

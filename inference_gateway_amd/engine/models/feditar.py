@@ -258,16 +258,16 @@ class DecayMemory(nn.Module):
 
 class ParallelMixer(nn.Module):
     """Two mixers read the same input; each output is RMS-normed over
-    the model width with its own plain weight, and the two are averaged."""
+    the model width with its own plain weight, and the two are averaged.
+    `left` and `right` are any two mixer modules whose cache_spec() is a
+    list of buffers and whose forward is (h, batch, buffers)."""
 
-    def __init__(self, hidden: int, spec: ParallelMixerSpec, eps: float,
-                 name: str, device, dtype):
+    def __init__(self, hidden: int, left: nn.Module, right: nn.Module,
+                 eps: float, name: str, device):
         super().__init__()
         self.eps = eps
-        self.left = SoftcapAttention(hidden, spec.left, name + ".left",
-                                     device, dtype)
-        self.right = DecayMemory(hidden, spec.right, eps, name + ".right",
-                                 device, dtype)
+        self.left, self.right = left, right
+        self.n_left = len(left.cache_spec())
         self.left_out = _param(1.0 + _rand((hidden,), device, torch.float32,
                                            name + ".left.out", 5.0))
         self.right_out = _param(1.0 + _rand((hidden,), device,
@@ -278,8 +278,8 @@ class ParallelMixer(nn.Module):
         return ("group", self.left.cache_spec() + self.right.cache_spec())
 
     def forward(self, h, fb: ForwardBatch, cache):
-        a = self.left(h, fb, cache[:2])
-        b = self.right(h, fb, cache[2:])
+        a = self.left(h, fb, cache[:self.n_left])
+        b = self.right(h, fb, cache[self.n_left:])
         return ops.rmsnorm_pair_mean(a, b, self.left_out, self.right_out,
                                      self.eps)
 
@@ -309,8 +309,11 @@ class FeditarLayer(nn.Module):
         elif spec.type == "mamba2":
             self.mixer = Mamba2Mixer(D, spec.mixer, eps, name, device, dtype)
         elif spec.type == "parallel":
-            self.mixer = ParallelMixer(D, spec.mixer, eps, name, device,
-                                       dtype)
+            self.mixer = ParallelMixer(
+                D, SoftcapAttention(D, spec.mixer.left, name + ".left",
+                                    device, dtype),
+                DecayMemory(D, spec.mixer.right, eps, name + ".right",
+                            device, dtype), eps, name, device)
         else:
             raise ValueError(f"layer {i}: unknown mixer {spec.type!r}")
         if spec.mlp is None:

@@ -8,8 +8,8 @@ from pathlib import Path
 
 import torch
 
-from ..config import (FedatarConfig, FeditarConfig, MekevikConfig,
-                      ModelConfig)
+from ..config import (BozolornConfig, FedatarConfig, FeditarConfig,
+                      MekevikConfig, ModelConfig)
 
 
 def build_model(model_cfg, device, dtype):
@@ -20,6 +20,8 @@ def build_model(model_cfg, device, dtype):
         from .mekevik import MekevikForCausalLM as cls
     elif isinstance(model_cfg, FeditarConfig):
         from .feditar import FeditarForCausalLM as cls
+    elif isinstance(model_cfg, BozolornConfig):
+        from .bozolorn import BozolornForCausalLM as cls
     elif model_cfg.is_moe:
         from .mixtral import MixtralForCausalLM as cls
     else:
@@ -60,6 +62,10 @@ def model_config_from_dir(path: str):
         return FeditarConfig.from_dict(
             cfg, name=Path(path).name or "feditar",
             shapes=safetensors_shapes(path))
+    if cfg.get("architecture") == "Bozolorn":
+        return BozolornConfig.from_dict(
+            cfg, name=Path(path).name or "bozolorn",
+            shapes=safetensors_shapes(path))
     if cfg.get("architecture") == "Fedatar":
         return FedatarConfig.from_dict(
             cfg, name=Path(path).name or "fedatar",
@@ -75,10 +81,13 @@ def is_recurrent(model_cfg) -> bool:
     a shared prefix's end is not stored)."""
     if isinstance(model_cfg, FeditarConfig):
         return True     # every mixer and the embedding keep slot state
+    if isinstance(model_cfg, BozolornConfig):
+        # the delta-rule half of a parallel mixer keeps slot state
+        return any(l.type == "parallel" for l in model_cfg.layers)
     return isinstance(model_cfg, FedatarConfig) and any(
         l.type == "mingru" for l in model_cfg.layers)
 
 
 __all__ = ["build_model", "model_config_from_dir", "safetensors_shapes",
            "is_recurrent", "ModelConfig", "FedatarConfig", "MekevikConfig",
-           "FeditarConfig"]
+           "FeditarConfig", "BozolornConfig"]

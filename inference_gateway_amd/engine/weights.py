@@ -483,6 +483,84 @@ def load_feditar_weights(model, path: str) -> int:
     return n
 
 
+def load_bozolorn_weights(model, path: str) -> int:
+    """Load a Bozolorn checkpoint: tensors `embed`, `side.embed`,
+    `l<i>.norm1|norm1b|norm2|norm2b`, `l<i>.mix.*` per mixer kind,
+    `l<i>.mlp.{router,correction}` and `l<i>.mlp.e<j>.{gate,up,down}`,
+    `l<i>.side.{gate,proj,norm}`, `final.norm`, `head`.  The engine's
+    layouts are assembled here: q|k|v|g (q|g for a layer that borrows its
+    keys and values) stacked for the attention input GEMM; q|k|v with
+    their biases for the rotated attention; q|k|v|g and the three
+    convolution filters stacked for the delta-rule memory, its step and
+    write-strength rows stacked apart in fp32 and its per-head norm
+    weight repeated for every head; experts stacked K-major with gate|up
+    side by side."""
+    sh = _Shards(path)
+    cfg = model.cfg
+    n = 0
+
+    def put(param, src, what):
+        nonlocal n
+        _copy(param, src, what)
+        n += 1
+
+    def cat(prefix, names, suffix=""):
+        return torch.cat([sh.full(prefix + c + suffix) for c in names], 0)
+
+    put(model.embed, sh.full("embed"), "embed")
+    if model.side_embed is not None:
+        put(model.side_embed, sh.full("side.embed"), "side.embed")
+    for i, (spec, layer) in enumerate(zip(cfg.layers, model.layers)):
+        p = f"l{i}."
+        put(layer.norm1_w, sh.full(p + "norm1"), p + "norm1")
+        put(layer.norm1b_w, sh.full(p + "norm1b"), p + "norm1b")
+        mx, m = layer.mixer, p + "mix."
+        if spec.type == "attention":
+            rows = "qkvg" if mx.owns_kv else "qg"
+            put(mx.qkvg, cat(m, rows), m + "|".join(rows))
+            put(mx.o, sh.full(m + "o"), m + "o")
+        else:
+            a, ml = mx.left, m + "left."
+            put(a.qkv, cat(ml, "qkv"), ml + "q|k|v")
+            put(a.qkv_b, cat(ml, "qkv", ".b"), ml + "q|k|v.b")
+            put(a.qnorm_w, sh.full(ml + "q.norm"), ml + "q.norm")
+            put(a.knorm_w, sh.full(ml + "k.norm"), ml + "k.norm")
+            put(a.o, sh.full(ml + "o"), ml + "o")
+            b, mr = mx.right, m + "right."
+            put(b.qkvg, cat(mr, "qkvg"), mr + "q|k|v|g")
+            put(b.conv_w, cat(mr, "qkv", ".conv"), mr + "q|k|v.conv")
+            put(b.ab_w, cat(mr, "ab"), mr + "a|b")
+            put(b.a_log, sh.full(mr + "A_log"), mr + "A_log")
+            put(b.dt_bias, sh.full(mr + "dt_bias"), mr + "dt_bias")
+            put(b.norm_w, sh.full(mr + "norm").repeat(spec.mixer.right.heads),
+                mr + "norm")
+            put(b.o, sh.full(mr + "o"), mr + "o")
+            put(mx.left_out, sh.full(ml + "out"), ml + "out")
+            put(mx.right_out, sh.full(mr + "out"), mr + "out")
+        if spec.mlp is not None:
+            put(layer.norm2_w, sh.full(p + "norm2"), p + "norm2")
+            put(layer.norm2b_w, sh.full(p + "norm2b"), p + "norm2b")
+            f, ff = layer.mlp, p + "mlp."
+            put(f.router_w, sh.full(ff + "router"), ff + "router")
+            put(f.correction, sh.full(ff + "correction"), ff + "correction")
+            E = spec.mlp.experts
+            put(f.up_t, torch.stack([
+                torch.cat([sh.full(ff + f"e{e}.gate"),
+                           sh.full(ff + f"e{e}.up")], 0).t()
+                for e in range(E)]), ff + "e*.gate|up")
+            put(f.down_t, torch.stack(
+                [sh.full(ff + f"e{e}.down").t() for e in range(E)]),
+                ff + "e*.down")
+        if layer.side is not None:
+            sd = p + "side."
+            put(layer.side.gate, sh.full(sd + "gate"), sd + "gate")
+            put(layer.side.proj, sh.full(sd + "proj"), sd + "proj")
+            put(layer.side.norm_w, sh.full(sd + "norm"), sd + "norm")
+    put(model.final_norm_w, sh.full("final.norm"), "final.norm")
+    put(model.head, sh.full("head"), "head")
+    return n
+
+
 def _is_gguf(path: str) -> bool:
     p = Path(path)
     if p.is_file():
@@ -508,6 +586,8 @@ def load_weights(model, path: str) -> int:
         return load_mekevik_weights(model, path)
     if getattr(model.cfg, "architecture", "") == "Feditar":
         return load_feditar_weights(model, path)
+    if getattr(model.cfg, "architecture", "") == "Bozolorn":
+        return load_bozolorn_weights(model, path)
     if getattr(model.cfg, "is_moe", False):
         return load_mixtral_weights(model, path)
     return load_llama_weights(model, path)

@@ -590,11 +590,10 @@ def gated_act(gate_up, mode: int, limit: float = 0.0, alpha: float = 1.0):
     GATED_ACT_SILU silu(g) * u; GATED_ACT_CLAMPED with g' = min(g, limit),
     u' = clamp(u, -limit, limit): g' * sigmoid(alpha g') * (u' + 1)."""
     if gate_up.is_cuda:
-        _require_hybrid()
         f = gate_up.shape[-1] // 2
         out = torch.empty((*gate_up.shape[:-1], f), dtype=gate_up.dtype,
                           device=gate_up.device)
-        _hybrid.gated_act(out, gate_up, mode, limit, alpha)
+        _shared_ext("gated_act")(out, gate_up, mode, limit, alpha)
         return out
     return torch_ref.gated_act_ref(gate_up, mode, limit, alpha)
 
@@ -777,12 +776,18 @@ def softcap_attention(q, kcache, vcache, block_table, row_seq, positions,
                       scale: float, softcap: float = 0.0,
                       temp_coef: float = 0.0, temp_every: int = 1,
                       window: int = 0, num_prefill_rows: int = 0,
-                      prefill_seq_lens=None, seq_cu=None, seq_start=None):
+                      prefill_seq_lens=None, seq_cu=None, seq_start=None,
+                      slopes=None, chunk: int = 0, sinks=None, gate=None):
     """Causal softmax attention over paged keys/values with grouped
     heads and separate key and value widths.  score = (q . k) * scale *
     (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)), squashed by
     softcap * tanh(. / softcap) when softcap > 0; window > 0 keeps the
-    last `window` keys.  q [T, H*N] (strided ok) -> [T, H*P].  Rows [0,
+    last `window` keys.  Optional: slopes [H] fp32 take slope_h * (p - j)
+    off the score of key j; chunk > 0 keeps only the keys from floor(p /
+    chunk) * chunk on; sinks [H] fp32 add exp(sink_h) to the softmax
+    denominator (a key with that score and no value); gate [T, H*P]
+    (strided rows ok) multiplies the result by sigmoid(gate).
+    q [T, H*N] (strided ok) -> [T, H*P].  Rows [0,
     num_prefill_rows) are prompt portions (prefill_seq_lens = python row
     counts of the first sequences), the rest single decoded tokens;
     seq_cu / seq_start describe the sequences (needed by the tile
@@ -801,15 +806,136 @@ def softcap_attention(q, kcache, vcache, block_table, row_seq, positions,
             if _recurrent.softcap_attention_mfma(
                     out, q, kcache, vcache, block_table, seq_cu, seq_start,
                     tseq, toff, dec, scale, softcap, temp_coef, temp_every,
-                    window):
+                    window, slopes, chunk, sinks, gate):
                 return out
         _recurrent.softcap_attention(out, q, kcache, vcache, block_table,
                                      row_seq, positions, scale, softcap,
-                                     temp_coef, temp_every, window)
+                                     temp_coef, temp_every, window, slopes,
+                                     chunk, sinks, gate)
         return out
     return recurrent_ref.softcap_attention_ref(
         q, kcache, vcache, block_table, row_seq, positions, scale, softcap,
-        temp_coef, temp_every, window)
+        temp_coef, temp_every, window, slopes, chunk, sinks, gate)
+
+
+def qk_norm_rope_append(proj, positions, slot_mapping, kcache, vcache,
+                        qnorm_w, knorm_w, inv_freq, mag: float, eps: float,
+                        heads: int, kv_heads: int, dim: int, vdim: int):
+    """Post-processing of a fused projection [T, heads*dim | kv_heads*dim
+    | kv_heads*vdim | ...] (strided rows ok): per-head RMS norm of the
+    queries and keys (weights [dim] fp32 shared by the heads; None = no
+    norm), interleaved-pair rotation of each head's first
+    2*len(inv_freq) entries by position * inv_freq (fp32 angles, cos and
+    sin times `mag`; inv_freq None = no rotation), keys and values
+    appended to the paged caches [blocks, kv_heads, block, dim | vdim].
+    Returns the queries [T, heads*dim]."""
+    if proj.is_cuda:
+        _require_recurrent()
+        q = torch.empty((proj.shape[0], heads * dim), dtype=proj.dtype,
+                        device=proj.device)
+        _recurrent.qk_norm_rope_append(q, proj, positions, slot_mapping,
+                                       kcache, vcache, qnorm_w, knorm_w,
+                                       inv_freq, mag, eps, heads, kv_heads,
+                                       dim, vdim)
+        return q
+    return recurrent_ref.qk_norm_rope_append_ref(
+        proj, positions, slot_mapping, kcache, vcache, qnorm_w, knorm_w,
+        inv_freq, mag, eps, heads, kv_heads, dim, vdim)
+
+
+def decay_beta_gates(pre, a_log, dt_bias):
+    """Gates of a delta-rule memory from fp32 pre-activations [T, 2H]
+    (step | write strength): decay = exp(-exp(a_log) * softplus(step +
+    dt_bias)), beta = sigmoid(write strength).  Returns fp32 (decay,
+    beta), each [T, H]."""
+    if pre.is_cuda:
+        _require_recurrent()
+        T, H = pre.shape[0], pre.shape[1] // 2
+        out = torch.empty((2, T, H), dtype=torch.float32, device=pre.device)
+        _recurrent.decay_beta_gates(out, pre, a_log, dt_bias)
+        return out[0], out[1]
+    return recurrent_ref.decay_beta_gates_ref(pre, a_log, dt_bias)
+
+
+def delta_scan(q, k, v, decay, beta, state, seq_cu, seq_start, seq_slots,
+               seq_rows, unit_eps: float = 0.0, qscale: float = 1.0):
+    """Gated delta-rule memory per (sequence, head), S [N, P] fp32 in
+    state [slots, H*N*P].  Per row, in this order: S <- a_t S; u = b_t
+    (v_t - S^T k_t); S <- S + k_t u^T; o_t = S^T q_t.  With unit_eps > 0
+    q and k are first scaled to unit length per head (x / sqrt(sum x^2 +
+    unit_eps)); q is multiplied by qscale.  q, k [T, G, N] (strided ok;
+    head h reads group h // (H/G)), v [T, H, P], decay and beta fp32 [T,
+    H].  Returns o fp32 [T, H, P].  seq_rows: python row counts."""
+    if v.is_cuda:
+        _require_recurrent()
+        T, H, P = v.shape
+        out = torch.empty((T, H, P), dtype=torch.float32, device=v.device)
+        _recurrent.delta_scan(out, q, k, v, decay, beta, state, seq_cu,
+                              seq_start, seq_slots, unit_eps, qscale)
+        return out
+    return recurrent_ref.delta_scan_ref(q, k, v, decay, beta, state, seq_cu,
+                                        seq_start, seq_slots, unit_eps,
+                                        qscale)
+
+
+def moe_group_route(logits, correction, top_k: int, groups: int, keep: int,
+                    capacity: int = 0):
+    """Sigmoid router with a selection-only correction and expert
+    groups: logits [T, E] fp32, correction [E] fp32 -> (weights [T, K]
+    fp32 = sigmoid(logit) of the chosen experts, not renormalised; expert
+    ids [T, K] int32; padded rows [T*K] int64 or None).  Choice score =
+    sigmoid(logit) + correction; the E experts form `groups` equal runs
+    of neighbours, a group scores the sum of its two best choice scores
+    and only the `keep` best groups can be chosen from.  With capacity >
+    0 (>= T) the padded-dispatch row of every assignment, expert *
+    capacity + rank, comes from the same launch.  E <= 64 on the GPU
+    kernel."""
+    if logits.is_cuda and logits.shape[1] <= 64:
+        _require_recurrent()
+        T, E = logits.shape
+        w = torch.empty((T, top_k), dtype=torch.float32,
+                        device=logits.device)
+        idx = torch.empty((T, top_k), dtype=torch.int32,
+                          device=logits.device)
+        dst = counts = None
+        if capacity > 0:
+            dst = torch.empty(T * top_k, dtype=torch.int64,
+                              device=logits.device)
+            counts = torch.zeros(E, dtype=torch.int32, device=logits.device)
+        _recurrent.moe_group_route(w, idx, logits, correction, dst, counts,
+                                   capacity, groups, keep)
+        return w, idx, dst
+    w, idx = recurrent_ref.moe_group_route_ref(logits, correction, top_k,
+                                               groups, keep)
+    return w, idx, None
+
+
+def add_normed_rmsnorm(residual, delta, w_post, w_pre, eps: float,
+                       out_dtype):
+    """Sandwich-norm step: residual [T, D] fp32 += rmsnorm(delta) *
+    w_post (in place; delta None = nothing added), then returns
+    rmsnorm(residual) * w_pre in out_dtype (w_pre None: the residual
+    itself in out_dtype).  Weights fp32 [D]."""
+    if residual.is_cuda:
+        _require_recurrent()
+        out = torch.empty(residual.shape, dtype=out_dtype,
+                          device=residual.device)
+        _recurrent.add_normed_rmsnorm(out, residual, delta, w_post, w_pre,
+                                      eps)
+        return out
+    return recurrent_ref.add_normed_rmsnorm_ref(residual, delta, w_post,
+                                                w_pre, eps, out_dtype)
+
+
+def gelu_mul_rows(z, table, tokens, col0: int):
+    """gelu_tanh(z [T, W]) * table[tokens, col0 : col0 + W] (table rows
+    gathered by token id)."""
+    if z.is_cuda:
+        _require_recurrent()
+        out = torch.empty_like(z)
+        _recurrent.gelu_mul_rows(out, z, table, tokens, col0)
+        return out
+    return recurrent_ref.gelu_mul_rows_ref(z, table, tokens, col0)
 
 
 def rmsnorm_pair_mean(a, b, wa, wb, eps: float):

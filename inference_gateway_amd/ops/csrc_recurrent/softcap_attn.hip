@@ -5,9 +5,13 @@
 //   score_j = (q[t,h] . K_j[g]) * scale * temp(p),   lo <= j <= p
 //   temp(p) = 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)
 //   score_j <- softcap * tanh(score_j / softcap)      (softcap > 0)
+//   score_j <- score_j - slope[h] * (p - j)            (slopes given)
 //   out[t,h] = sum_j softmax_j(score) V_j[g]          [P]
 //
-// lo = max(0, p - window + 1) with a window, 0 without.  Keys are
+// lo = max(0, p - window + 1) with a window, 0 without; with chunk > 0 also
+// lo >= floor(p / chunk) * chunk (keys of the row's own position chunk).
+// With sinks, exp(sink[h]) joins the softmax denominator (a key of that
+// score without a value); with a gate, out[t,h] *= sigmoid(gate[t,h]).  Keys are
 // [blocks, G, block, N], values [blocks, G, block, P]; N and P need not be
 // equal.  Scores, probabilities and the accumulator are fp32.
 //
@@ -26,7 +30,9 @@ __global__ __launch_bounds__(64) void softcap_attention_rows_kernel(
     const int32_t* __restrict__ block_table, int max_blocks,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ positions,
     float scale, float softcap, float temp_coef, int temp_every, int window,
-    int H, int G, int N, int P, int block_size) {
+    const float* __restrict__ slopes, int chunk,
+    const float* __restrict__ sinks, const T* __restrict__ gate,
+    int64_t gate_stride, int H, int G, int N, int P, int block_size) {
   extern __shared__ float lds[];
   float* ql = lds;                            // [N], pre-scaled
   float* p_lds = lds + N;                     // [64]
@@ -35,7 +41,9 @@ __global__ __launch_bounds__(64) void softcap_attention_rows_kernel(
   const int g = h / (H / G);
   const int pos = positions[t];
   const int32_t* bt = block_table + (int64_t)row_seq[t] * max_blocks;
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, pos / chunk * chunk);
+  const float slope = slopes ? slopes[h] : 0.0f;
   const float temp =
       1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f);
   const float qs = scale * temp;
@@ -59,6 +67,7 @@ __global__ __launch_bounds__(64) void softcap_attention_rows_kernel(
       float a = 0.0f;
       for (int d = 0; d < N; ++d) a += ql[d] * Act<T>::ld(row + d);
       s = softcap > 0.0f ? softcap * tanhf(a * inv_cap) : a;
+      s -= slope * (float)(pos - j);
     }
     const float m_new = fmaxf(m, wave_reduce_max(s));
     const float corr = expf(m - m_new);
@@ -82,12 +91,20 @@ __global__ __launch_bounds__(64) void softcap_attention_rows_kernel(
       }
     }
   }
+  // the sink's term relative to the running maximum (an overflow to
+  // infinity gives the right limit, an all-zero row)
+  if (sinks) l += expf(sinks[h] - m);
   const float inv = 1.0f / l;
   T* o = out + ((int64_t)t * H + h) * P;
+  const T* gt = gate ? gate + (int64_t)t * gate_stride + h * P : nullptr;
 #pragma unroll
   for (int i = 0; i < NACC; ++i) {
     const int d = lane + 64 * i;
-    if (d < P) Act<T>::st(o + d, acc[i] * inv);
+    if (d < P) {
+      float y = acc[i] * inv;
+      if (gt) y *= sigmoid_f32(Act<T>::ld(gt + d));
+      Act<T>::st(o + d, y);
+    }
   }
 }
 
@@ -95,7 +112,10 @@ void softcap_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kcache,
                        torch::Tensor vcache, torch::Tensor block_table,
                        torch::Tensor row_seq, torch::Tensor positions,
                        double scale, double softcap, double temp_coef,
-                       int64_t temp_every, int64_t window) {
+                       int64_t temp_every, int64_t window,
+                       c10::optional<torch::Tensor> slopes, int64_t chunk,
+                       c10::optional<torch::Tensor> sinks,
+                       c10::optional<torch::Tensor> gate) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 2 && q.stride(1) == 1);
   TORCH_CHECK(kcache.is_contiguous() && kcache.dim() == 4 &&
               vcache.is_contiguous() && vcache.dim() == 4 &&
@@ -113,7 +133,17 @@ void softcap_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kcache,
   TORCH_CHECK(row_seq.dtype() == torch::kInt32 && row_seq.numel() == T);
   TORCH_CHECK(positions.dtype() == torch::kInt32 && positions.numel() == T);
   TORCH_CHECK(P <= 1024, "value width above 1024 is not supported");
-  TORCH_CHECK(temp_every >= 1);
+  TORCH_CHECK(temp_every >= 1 && chunk >= 0);
+  if (slopes.has_value())
+    TORCH_CHECK(slopes->dtype() == torch::kFloat32 &&
+                slopes->is_contiguous() && slopes->numel() == H);
+  if (sinks.has_value())
+    TORCH_CHECK(sinks->dtype() == torch::kFloat32 && sinks->is_contiguous() &&
+                sinks->numel() == H);
+  if (gate.has_value())
+    TORCH_CHECK(gate->dtype() == q.dtype() && gate->dim() == 2 &&
+                gate->stride(1) == 1 && gate->size(0) == T &&
+                gate->size(1) == (int64_t)H * P);
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
   const size_t shmem = (size_t)(N + 128) * sizeof(float);
@@ -127,7 +157,12 @@ void softcap_attention(torch::Tensor out, torch::Tensor q, torch::Tensor kcache,
       (const int32_t*)block_table.data_ptr(), (int)block_table.size(1),      \
       (const int32_t*)row_seq.data_ptr(),                                    \
       (const int32_t*)positions.data_ptr(), (float)scale, (float)softcap,    \
-      (float)temp_coef, (int)temp_every, (int)window, H, G, N, P, bs)
+      (float)temp_coef, (int)temp_every, (int)window,                        \
+      slopes.has_value() ? (const float*)slopes->data_ptr() : nullptr,       \
+      (int)chunk,                                                            \
+      sinks.has_value() ? (const float*)sinks->data_ptr() : nullptr,         \
+      gate.has_value() ? (const act_t*)gate->data_ptr() : nullptr,           \
+      gate.has_value() ? (int64_t)gate->stride(0) : 0, H, G, N, P, bs)
   IGW_DISPATCH_ACT(q, {
     if (nacc <= 1) LAUNCH_ROWS(1);
     else if (nacc <= 2) LAUNCH_ROWS(2);

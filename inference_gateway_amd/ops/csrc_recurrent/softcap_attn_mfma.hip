@@ -9,7 +9,11 @@
 //     to the template's NP / PP (N, P multiples of 8);
 //   * any page size;
 //   * score = q.k * scale * temp(position), then cap * tanh(. / cap);
-//   * an optional sliding window;
+//   * an optional sliding window, an optional restriction to the row's
+//     own chunk of positions, an optional linear distance bias per head
+//     (slope * (row position - key position) is taken off the score), an
+//     optional sink term per head in the softmax denominator and an
+//     optional sigmoid output gate;
 //   * two row maps.  Prompt tiles: rows are 64 consecutive tokens of one
 //     head (grid = tiles x heads).  Decoded rows (HEADS_ROWS): the rows of
 //     a tile are the query heads that share one key/value head, so every
@@ -57,7 +61,10 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
     const int32_t* __restrict__ seq_cu, const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_off,
     int H, int G, int N, int P, int BS, float scale, float softcap,
-    float temp_coef, int temp_every, int window) {
+    float temp_coef, int temp_every, int window,
+    const float* __restrict__ slopes, int chunk,
+    const float* __restrict__ sinks, const uint16_t* __restrict__ gate,
+    int64_t gate_rs) {
   constexpr int BM = SA_BM, BN = SA_BN;
   constexpr int KROWB = NP * 2;          // bytes per staged Q / K row
   // K tile (shared with the Q staging) | V^T tile | per-wave P tiles
@@ -124,8 +131,8 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
           swz<KROWB>(row, (kk * 32 + frag_k8) * 2));
   }
 
-  float m[4], l[4], rscale[4];
-  int qpos[4];
+  float m[4], l[4], rscale[4], slope[4];
+  int qpos[4], klo[4];
   float4v acc_o[PP / 16];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -134,6 +141,13 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
     qpos[r] = HEADS_ROWS ? P0 : P0 + qoff + wave * 16 + crow0 + r;
     rscale[r] = scale * (1.0f + temp_coef * logf((float)((qpos[r] + 1) /
                                                          temp_every) + 1.0f));
+    // first visible key of the row: window and position chunk
+    klo[r] = window > 0 ? qpos[r] - window + 1 : 0;
+    if (chunk > 0) klo[r] = max(klo[r], qpos[r] / chunk * chunk);
+    const int head_r =
+        HEADS_ROWS ? kvh * rep + min(wave * 16 + crow0 + r, rep - 1)
+                   : (int)blockIdx.y;
+    slope[r] = slopes ? slopes[head_r] : 0.0f;
   }
 #pragma unroll
   for (int nt = 0; nt < PP / 16; ++nt) acc_o[nt] = {0.f, 0.f, 0.f, 0.f};
@@ -142,8 +156,9 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
   // keys [kfirst, kend): up to the tile's last row, from its first row's
   // window start
   const int kend = HEADS_ROWS ? KVL : min(KVL, P0 + qoff + BM);
-  const int kfirst =
-      window > 0 ? max(0, P0 + qoff - window + 1) / BN * BN : 0;
+  int kfirst = window > 0 ? max(0, P0 + qoff - window + 1) : 0;
+  if (chunk > 0) kfirst = max(kfirst, (P0 + qoff) / chunk * chunk);
+  kfirst = kfirst / BN * BN;
 
   // the next K/V tile travels in registers while the current one is used
   // (a second tile in flight costs more in occupancy than it hides)
@@ -228,13 +243,14 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
     float pmax[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int lo = window > 0 ? qpos[r] - window + 1 : 0;
+      const int lo = klo[r];
       float mx = -INFINITY;
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const int kpos = kbase + nt * 16 + ccol;
         float s = acc_s[nt][r] * rscale[r];
         if (softcap > 0.0f) s = softcap * tanh_fast(s * inv_cap);
+        s -= slope[r] * (float)(qpos[r] - kpos);
         if (kpos > qpos[r] || kpos >= KVL || kpos < lo) s = -INFINITY;
         acc_s[nt][r] = s;
         mx = fmaxf(mx, s);
@@ -289,12 +305,20 @@ __global__ __launch_bounds__(256, 2) void softcap_attention_mfma_kernel(
     if (row >= nrows) continue;
     const int64_t tok = HEADS_ROWS ? q0 : q0 + qoff + row;
     const int head = HEADS_ROWS ? kvh * rep + row : blockIdx.y;
-    const float inv = 1.0f / l[r];
+    // the sink's term relative to the running maximum (an overflow to
+    // infinity gives the right limit, an all-zero row)
+    const float lsum = sinks ? l[r] + __expf(sinks[head] - m[r]) : l[r];
+    const float inv = 1.0f / lsum;
     uint16_t* o = out + (tok * H + head) * P;
+    const uint16_t* gt = gate ? gate + tok * gate_rs + head * P : nullptr;
 #pragma unroll
     for (int nt = 0; nt < PP / 16; ++nt) {
       const int c = nt * 16 + ccol;
-      if (c < P) o[c] = f32_to_bf16(acc_o[nt][r] * inv);
+      if (c < P) {
+        float y = acc_o[nt][r] * inv;
+        if (gt) y *= sigmoid_fast(bf16_to_f32(gt[c]));
+        o[c] = f32_to_bf16(y);
+      }
     }
   }
 }
@@ -310,7 +334,10 @@ bool softcap_attention_mfma(torch::Tensor out, torch::Tensor q,
                             torch::Tensor seq_start, torch::Tensor tile_seq,
                             torch::Tensor tile_off, torch::Tensor dec_seq,
                             double scale, double softcap, double temp_coef,
-                            int64_t temp_every, int64_t window) {
+                            int64_t temp_every, int64_t window,
+                            c10::optional<torch::Tensor> slopes,
+                            int64_t chunk, c10::optional<torch::Tensor> sinks,
+                            c10::optional<torch::Tensor> gate) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 2 && q.stride(1) == 1);
   if (q.scalar_type() != torch::kBFloat16) return false;
   TORCH_CHECK(kcache.is_contiguous() && kcache.dim() == 4 &&
@@ -337,7 +364,17 @@ bool softcap_attention_mfma(torch::Tensor out, torch::Tensor q,
   TORCH_CHECK(tile_seq.dtype() == torch::kInt32 &&
               tile_off.dtype() == torch::kInt32 &&
               tile_off.numel() == ntile && dec_seq.dtype() == torch::kInt32);
-  TORCH_CHECK(temp_every >= 1);
+  TORCH_CHECK(temp_every >= 1 && chunk >= 0);
+  if (slopes.has_value())
+    TORCH_CHECK(slopes->dtype() == torch::kFloat32 &&
+                slopes->is_contiguous() && slopes->numel() == H);
+  if (sinks.has_value())
+    TORCH_CHECK(sinks->dtype() == torch::kFloat32 && sinks->is_contiguous() &&
+                sinks->numel() == H);
+  if (gate.has_value())
+    TORCH_CHECK(gate->dtype() == q.dtype() && gate->dim() == 2 &&
+                gate->stride(1) == 1 && gate->size(0) == T &&
+                gate->size(1) == (int64_t)H * P);
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
 #define LAUNCH_SA(NPV, PPV, HR, GRID, TSEQ)                                   \
   hipLaunchKernelGGL(                                                         \
@@ -349,7 +386,12 @@ bool softcap_attention_mfma(torch::Tensor out, torch::Tensor q,
       (const int32_t*)seq_cu.data_ptr(), (const int32_t*)seq_start.data_ptr(), \
       (const int32_t*)TSEQ.data_ptr(), (const int32_t*)tile_off.data_ptr(),   \
       H, G, N, P, BS, (float)scale, (float)softcap, (float)temp_coef,         \
-      (int)temp_every, (int)window)
+      (int)temp_every, (int)window,                                           \
+      slopes.has_value() ? (const float*)slopes->data_ptr() : nullptr,        \
+      (int)chunk,                                                             \
+      sinks.has_value() ? (const float*)sinks->data_ptr() : nullptr,          \
+      gate.has_value() ? (const uint16_t*)gate->data_ptr() : nullptr,         \
+      gate.has_value() ? (int64_t)gate->stride(0) : 0)
 #define LAUNCH_SA_SIZES(HR, GRID, TSEQ)                                       \
   do {                                                                        \
     if (N <= 64 && P <= 64) LAUNCH_SA(64, 64, HR, GRID, TSEQ);                \

@@ -209,12 +209,17 @@ def append_paged_kv_ref(k, v, kcache, vcache, slot_mapping):
 
 def softcap_attention_ref(q, kcache, vcache, block_table, row_seq,
                           positions, scale, softcap, temp_coef, temp_every,
-                          window):
+                          window, slopes=None, chunk=0, sinks=None,
+                          gate=None):
     """Causal softmax attention of every row against its sequence's
     paged keys 0..position (the last `window` of them when window > 0).
     score = (q . k) * scale * temp(p), temp(p) = 1 + temp_coef *
     ln(floor((p + 1) / temp_every) + 1); then softcap * tanh(score /
-    softcap) when softcap > 0.  q [T, H*N] -> [T, H*P]."""
+    softcap) when softcap > 0.  slopes [H]: slope_h * (p - j) is taken
+    off the score of key j.  chunk > 0: only keys from floor(p / chunk) *
+    chunk on.  sinks [H]: exp(sink_h) joins the softmax denominator (a
+    key with that score and no value).  gate [T, H*P]: the result is
+    multiplied by sigmoid(gate).  q [T, H*N] -> [T, H*P]."""
     nb, G, bs, N = kcache.shape
     P = vcache.shape[3]
     T = q.shape[0]
@@ -227,6 +232,8 @@ def softcap_attention_ref(q, kcache, vcache, block_table, row_seq,
     for t in range(T):
         p = pos_l[t]
         lo = max(0, p - window + 1) if window > 0 else 0
+        if chunk > 0:
+            lo = max(lo, p // chunk * chunk)
         j = torch.arange(lo, p + 1, device=q.device)
         blocks = block_table[seq_l[t]].to(torch.int64)[j // bs]
         kk = kcache[blocks, :, j % bs].float()      # [n, G, N]
@@ -237,8 +244,143 @@ def softcap_attention_ref(q, kcache, vcache, block_table, row_seq,
         s = torch.einsum("hn,jhn->hj", qf[t], kk) * (scale * temp)
         if softcap > 0:
             s = softcap * torch.tanh(s / softcap)
-        out[t] = torch.einsum("hj,jhp->hp", torch.softmax(s, -1), vv)
-    return out.reshape(T, H * P).to(q.dtype)
+        if slopes is not None:
+            s = s - slopes[:, None] * (p - j).float()[None, :]
+        if sinks is not None:
+            w = torch.softmax(torch.cat([s, sinks[:, None]], 1), -1)[:, :-1]
+        else:
+            w = torch.softmax(s, -1)
+        out[t] = torch.einsum("hj,jhp->hp", w, vv)
+    out = out.reshape(T, H * P)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(q.dtype)
+
+
+def qk_norm_rope_append_ref(proj, positions, slot_mapping, kcache, vcache,
+                            qnorm_w, knorm_w, inv_freq, mag, eps, heads,
+                            kv_heads, dim, vdim):
+    """proj [T, heads*dim | kv_heads*dim | kv_heads*vdim | ...]: every
+    query and key head is RMS-normed over its dim entries (weights [dim]
+    shared by the heads; None = no norm), then pairs (2i, 2i+1) of its
+    first 2*len(inv_freq) entries turn by position * inv_freq[i] with cos
+    and sin times `mag` (inv_freq None = no rotation).  Keys and values
+    go to the paged caches; the queries are returned [T, heads*dim]."""
+    T = proj.shape[0]
+    nq, nk = heads * dim, kv_heads * dim
+    q = proj[:, :nq].float().reshape(T, heads, dim)
+    k = proj[:, nq:nq + nk].float().reshape(T, kv_heads, dim)
+    v = proj[:, nq + nk:nq + nk + kv_heads * vdim]
+
+    def prep(x, w):
+        if w is not None:
+            x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w
+        if inv_freq is not None:
+            R = inv_freq.shape[0]
+            ang = positions.float()[:, None] * inv_freq.float()[None, :]
+            c = (torch.cos(ang) * mag)[:, None, :]
+            s = (torch.sin(ang) * mag)[:, None, :]
+            a, b = x[..., 0:2 * R:2], x[..., 1:2 * R:2]
+            rot = torch.stack([a * c - b * s, b * c + a * s], -1)
+            x = torch.cat([rot.reshape(T, x.shape[1], 2 * R),
+                           x[..., 2 * R:]], -1)
+        return x
+
+    q, k = prep(q, qnorm_w), prep(k, knorm_w)
+    append_paged_kv_ref(k.reshape(T, nk).to(proj.dtype), v, kcache, vcache,
+                        slot_mapping)
+    return q.reshape(T, nq).to(proj.dtype)
+
+
+def decay_beta_gates_ref(pre, a_log, dt_bias):
+    """pre [T, 2H] fp32 = (step | write-strength) pre-activations:
+    decay = exp(-exp(a_log) * softplus(step + dt_bias)), beta =
+    sigmoid(write-strength).  Returns fp32 ([T, H], [T, H])."""
+    H = pre.shape[1] // 2
+    dt = F.softplus(pre[:, :H] + dt_bias, threshold=40.0)
+    return torch.exp(-torch.exp(a_log) * dt), torch.sigmoid(pre[:, H:])
+
+
+def delta_scan_ref(q, k, v, decay, beta, state, seq_cu, seq_start,
+                   seq_slots, unit_eps, qscale):
+    """Gated delta-rule memory per (sequence, head), S [N, P] fp32 in
+    state [slots, H*N*P].  With unit_eps > 0, q and k are first scaled
+    to unit length per head, x / sqrt(sum x^2 + unit_eps); q is then
+    multiplied by qscale.  Per row, in this order:
+      S <- a_t S;  u = b_t (v_t - S^T k_t);  S <- S + k_t u^T;
+      o_t = S^T q_t.
+    q, k [T, G, N] (head h uses group h // (H/G)), v [T, H, P], decay and
+    beta fp32 [T, H]; returns o fp32 [T, H, P]."""
+    T, H, P = v.shape
+    G, N = q.shape[1], q.shape[2]
+    rep = H // G
+    qf, kf = q.float(), k.float()
+    if unit_eps > 0:
+        qf = qf * torch.rsqrt((qf * qf).sum(-1, keepdim=True) + unit_eps)
+        kf = kf * torch.rsqrt((kf * kf).sum(-1, keepdim=True) + unit_eps)
+    qf = (qf * qscale).repeat_interleave(rep, 1)
+    kf = kf.repeat_interleave(rep, 1)
+    vf = v.float()
+    out = torch.empty((T, H, P), dtype=torch.float32, device=v.device)
+    for r0, r1, st, sl in _seqs(seq_cu, seq_start, seq_slots):
+        if r1 == r0:
+            continue
+        S = (state[sl].view(H, N, P).clone() if st > 0 else torch.zeros(
+            (H, N, P), dtype=torch.float32, device=v.device))
+        for t in range(r0, r1):
+            S = S * decay[t][:, None, None]
+            u = beta[t][:, None] * (vf[t] - torch.einsum(
+                "hnp,hn->hp", S, kf[t]))
+            S = S + kf[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hnp,hn->hp", S, qf[t])
+        state[sl] = S.reshape(-1)
+    return out
+
+
+def moe_group_route_ref(logits, correction, top, groups, keep):
+    """logits [T, E] fp32 -> (weights [T, top] fp32, ids [T, top] int32).
+    Scores s = sigmoid(logits); choice scores c = s + correction.  The E
+    experts are `groups` equal runs of neighbours; a group's score is the
+    sum of its two largest choice scores (its only one when it has a
+    single expert) and only experts of the `keep` best groups can be
+    chosen; the `top` largest choice scores among them are taken and
+    weighted by their s (not renormalised)."""
+    T, E = logits.shape
+    s = torch.sigmoid(logits.float())
+    c = s + correction.float()
+    if groups > 1:
+        size = E // groups
+        cg = c.view(T, groups, size)
+        gscore = cg.topk(min(2, size), -1).values.sum(-1)
+        kept = gscore.topk(keep, -1).indices
+        mask = torch.zeros((T, groups), dtype=torch.bool,
+                           device=logits.device)
+        mask.scatter_(1, kept, True)
+        c = torch.where(mask[:, :, None], cg,
+                        torch.full_like(cg, float("-inf"))).reshape(T, E)
+    idx = c.topk(top, -1).indices
+    return s.gather(1, idx), idx.to(torch.int32)
+
+
+def add_normed_rmsnorm_ref(residual, delta, w_post, w_pre, eps, out_dtype):
+    """residual [T, D] fp32 += rmsnorm(delta) * w_post (in place; delta
+    None = nothing added); returns rmsnorm(residual) * w_pre in
+    out_dtype, or the residual itself in out_dtype when w_pre is None."""
+    if delta is not None:
+        d = delta.float()
+        residual += d * torch.rsqrt((d * d).mean(-1, keepdim=True)
+                                    + eps) * w_post
+    if w_pre is None:
+        return residual.to(out_dtype)
+    return (residual * torch.rsqrt((residual * residual).mean(
+        -1, keepdim=True) + eps) * w_pre).to(out_dtype)
+
+
+def gelu_mul_rows_ref(z, table, tokens, col0):
+    """gelu_tanh(z [T, W]) * table[tokens, col0 : col0 + W]."""
+    W = z.shape[1]
+    e = table[tokens.to(torch.int64), col0:col0 + W].float()
+    return (F.gelu(z.float(), approximate="tanh") * e).to(z.dtype)
 
 
 def rmsnorm_pair_mean_ref(a, b, wa, wb, eps):
