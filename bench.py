@@ -86,8 +86,8 @@ def parse_args():
                          "prints its own JSON object")
     ap.add_argument("--arch", type=str, default="fedatar",
                     help="design for --arch-compare: fedatar or mekevik "
-                         "(each beside Mixtral) or feditar (beside "
-                         "Fedatar)")
+                         "(each beside Mixtral), feditar (beside "
+                         "Fedatar) or bozolorn (beside Feditar)")
     ap.add_argument("--arch-size", type=str, default="2k",
                     help="layer shape for --arch-compare (2k | 4k)")
     ap.add_argument("--num-gpu-blocks", type=int, default=0,
@@ -518,6 +518,8 @@ def main() -> None:
             import bench_parallel as bench_hybrid
         elif args.arch == "feditar":
             import bench_recurrent as bench_hybrid
+        elif args.arch == "bozolorn":
+            import bench_bozolorn as bench_hybrid
         else:
             import bench_hybrid
 

@@ -279,3 +279,152 @@ def forward(W, cfg, tokens):
         taps.append(x.copy())
     logits = (rms_unit(x, eps) * W["final.norm"]) @ W["head"].T
     return logits, np.stack(taps)
+
+
+# ---------------------------------------------------------------------------
+# random checkpoints for the tests
+# ---------------------------------------------------------------------------
+def tensor_shapes(cfg):
+    """Tensor name -> shape of a checkpoint of this configuration."""
+    D, V = cfg["width"], cfg["vocab"]
+    L = len(cfg["layers"])
+    sh = {"embed": (V, D), "final.norm": (D,), "head": (V, D)}
+    side = (cfg.get("token_side") or {}).get("dim", 0)
+    if side:
+        sh["side.embed"] = (V, side * L)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        sh.update({p + "norm1": (D,), p + "norm1b": (D,)})
+        if l["type"] == "attention":
+            H, G, N, P = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            q = p + "mix."
+            sh.update({q + "q": (H * N, D), q + "g": (H * P, D),
+                       q + "o": (D, H * P)})
+            if m.get("kv_from") is None:
+                sh.update({q + "k": (G * N, D), q + "v": (G * P, D)})
+        else:
+            a, b = m["left"], m["right"]
+            H, G, N, P = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            q = p + "mix.left."
+            sh.update({q + "q": (H * N, D), q + "q.b": (H * N,),
+                       q + "k": (G * N, D), q + "k.b": (G * N,),
+                       q + "v": (G * P, D), q + "v.b": (G * P,),
+                       q + "q.norm": (N,), q + "k.norm": (N,),
+                       q + "o": (D, H * P), q + "out": (D,)})
+            H, G, N, P = b["heads"], b["kv_heads"], b["dim"], b["vdim"]
+            r = p + "mix.right."
+            sh.update({r + "q": (G * N, D), r + "q.conv": (G * N, b["conv"]),
+                       r + "k": (G * N, D), r + "k.conv": (G * N, b["conv"]),
+                       r + "v": (H * P, D), r + "v.conv": (H * P, b["conv"]),
+                       r + "b": (H, D), r + "a": (H, D), r + "A_log": (H,),
+                       r + "dt_bias": (H,), r + "norm": (P,),
+                       r + "g": (H * P, D), r + "o": (D, H * P),
+                       r + "out": (D,)})
+        f = l.get("mlp")
+        if f is not None:
+            E, ff = f["router"]["experts"], f["expert"]["ff"]
+            sh.update({p + "norm2": (D,), p + "norm2b": (D,),
+                       p + "mlp.router": (E, D), p + "mlp.correction": (E,)})
+            for e in range(E):
+                sh.update({p + f"mlp.e{e}.gate": (ff, D),
+                           p + f"mlp.e{e}.up": (ff, D),
+                           p + f"mlp.e{e}.down": (D, ff)})
+        if side:
+            sh.update({p + "side.gate": (side, D), p + "side.proj": (D, side),
+                       p + "side.norm": (D,)})
+    return sh
+
+
+def random_weights(cfg, seed=0):
+    """Random weights, rounded to bfloat16 (what a checkpoint stores),
+    as float64 arrays."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    W = {}
+    for name, shape in tensor_shapes(cfg).items():
+        x = torch.randn(shape, generator=g, dtype=torch.float32)
+        last = name.rsplit(".", 1)[-1]
+        if name == "embed":
+            x = x * 0.5 / cfg["embedding"]["scale"]
+        elif name == "side.embed":
+            x = x * 0.7
+        elif last in ("norm1", "norm2", "norm1b", "norm2b", "norm", "out"):
+            x = 1.0 + x * 0.2
+        elif last in ("A_log", "dt_bias"):
+            x = x * 0.7
+        elif last == "correction":
+            x = x * 0.3
+        elif last == "b" and len(shape) == 1:
+            x = x * 0.5
+        elif last == "conv":
+            x = x * 0.6
+        elif len(shape) == 2:
+            x = x * shape[1] ** -0.5 * (
+                3.0 if last in ("router", "a", "b") else 1.5)
+        W[name] = x.to(torch.bfloat16).double().numpy()
+    return W
+
+
+def save_checkpoint(path, cfg, W):
+    """config.json + model.safetensors (bfloat16) in `path`."""
+    import json
+    import os
+
+    import torch
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: torch.from_numpy(v).to(torch.bfloat16).contiguous()
+               for k, v in W.items()},
+              os.path.join(path, "model.safetensors"))
+    return str(path)
+
+
+def make_config(width, vocab, layers, side=0, scale=None, eps=1e-5):
+    cfg = {"architecture": "Bozolorn", "width": width, "vocab": vocab,
+           "norm": {"eps": eps},
+           "embedding": {"scale": scale or float(width) ** 0.5},
+           "layers": layers}
+    if side:
+        cfg["token_side"] = {"dim": side}
+    return cfg
+
+
+def moe_ff(experts, top, groups, keep, ff, limit):
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit},
+            "router": {"experts": experts, "top": top,
+                       "groups": {"count": groups, "keep": keep}}}
+
+
+def attention_layer(heads, kv_heads, dim, vdim, chunk, scale, mlp=None,
+                    kv_from=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+         "mask": {"size": chunk}, "scale": scale}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def rot(dims, base=10000.0, factor=None, original=None, fast=32.0,
+        slow=1.0):
+    r = {"dims": dims, "base": base}
+    if factor:
+        r["scaling"] = {"factor": factor, "original": original,
+                        "fast": fast, "slow": slow}
+    return r
+
+
+def parallel_layer(heads, kv_heads, dim, vdim, scale, rotary, d_heads,
+                   d_kv_heads, d_dim, d_vdim, conv, mlp=None):
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+            "scale": scale}
+    if rotary:
+        left["rot"] = rotary
+    return {"type": "parallel",
+            "mixer": {"left": left,
+                      "right": {"heads": d_heads, "kv_heads": d_kv_heads,
+                                "dim": d_dim, "vdim": d_vdim, "conv": conv}},
+            "mlp": mlp}
