@@ -113,6 +113,10 @@ __global__ __launch_bounds__(64 * DSCAN_MAX_WAVES) void delta_scan_kernel(
       }
       const float u = lds_b[t] * (vv - a * r);
       float o = 0.0f;
+      // the second pass must READ k again: if the compiler sees the same
+      // addresses it keeps the first pass's 128 loaded values in registers
+      // beside the state, which halves the occupancy
+      asm volatile("" : "+v"(k4), "+v"(q4));
 #pragma unroll
       for (int n4 = 0; n4 < NMAX / 4; ++n4) {
         const float4 qq = q4[n4], kk = k4[n4];

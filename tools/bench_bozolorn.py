@@ -211,6 +211,14 @@ def _kernels(sz):
         proj[:, H * N:H * N + G * N], proj[:, H * N + G * N:], kcs, vcs,
         slots))
     out["append_paged_kv"] = _entry(t, bytes_=T * G * (N + P) * 4.0)
+    if ops.HAS_HYBRID:
+        # the like kernel: Mekevik's norm over the whole q and k blocks +
+        # append (page-transposed values)
+        vct = torch.zeros(T // bs + 1, G, P, bs, device=dev, dtype=bf)
+        wq, wk = torch.ones(H * N, device=dev), torch.ones(G * N, device=dev)
+        t = _time(lambda: ops.qk_norm_append(proj, slots, kcs, vct, wq, wk,
+                                             None, 0.0, 1e-6, H, G, N, P))
+        out["qk_norm_append"] = _entry(t, bytes_=T * C * 4.0)
     CC = 2 * G * N + H * P
     pj = torch.randn(T, CC + H * P, device=dev, dtype=bf)
     cw = torch.randn(CC, 4, device=dev)
