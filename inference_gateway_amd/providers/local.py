@@ -229,8 +229,9 @@ class LocalProvider:
         weights = getattr(local_cfg, "weights_path", "") or None
         if local_cfg.model == "hf":
             # architecture straight from the checkpoint's config.json
-            # (HuggingFace Llama-family layouts, or the per-layer Fedatar
-            # and Mekevik designs, which name themselves in config.json)
+            # (HuggingFace Llama-family layouts, or the per-layer Fedatar,
+            # Mekevik, Feditar and Bozolorn designs, which name themselves
+            # in config.json)
             from ..engine.models.registry import model_config_from_dir
 
             preset = model_config_from_dir(weights)

@@ -704,6 +704,30 @@ def test_mixed_batches_against_each_alone(tmp_path, device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_first_tokens_in_used_slots(tmp_path, device):
+    """Requests of one, two and three tokens admitted into slots and
+    pages that longer requests have just left: the filter sees zeros
+    before position 0, the memory starts empty, the sink faces a single
+    key; a one-token request beside portions of others."""
+    cfg = cfg_small()
+    W = oracle.random_weights(cfg, 61)
+    eng = make_engine(tmp_path, cfg, W, device, blocks=24, slots=3)
+    for n in (19, 23, 11):                     # dirty every slot and page
+        replay_all(eng, toks(n, cfg["vocab"], 60 + n), [n])
+    reqs = [toks(n, cfg["vocab"], 70 + n) for n in (1, 2, 3)]
+    refs = [oracle.forward(W, cfg, t)[0] for t in reqs]
+    ids = [eng.open_stream() for _ in reqs]
+    out = eng.replay_step(
+        [(i, t[:2]) for i, t in zip(ids, reqs)],
+        {i: list(range(min(2, len(t)))) for i, t in zip(ids, reqs)})
+    close(out, np.concatenate([r[:2] for r in refs]), 2e-4)
+    out = eng.replay_step([(ids[2], reqs[2][2:])], {ids[2]: [0]})
+    close(out, refs[2][2:], 2e-4)
+    for i in ids:
+        eng.close_stream(i)
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_long_decode(tmp_path, device):
     cfg = cfg_ones()
     W = oracle.random_weights(cfg, 16)
