@@ -24,8 +24,15 @@ namespace igw {
 constexpr int DSCAN_CHUNK = 16;  // rows staged per pass
 constexpr int DSCAN_MAX_WAVES = 4;
 
-template <typename T, int NMAX>
-__global__ __launch_bounds__(64 * DSCAN_MAX_WAVES) void delta_scan_kernel(
+// MINB = workgroups per compute unit the register budget must allow.
+// Decoded rows (one row per sequence: load the state, one update, store it)
+// are latency-bound and gain from three waves per SIMD (168 registers at
+// 128 key entries: 144 -> 99 us for 256 sequences of 16 heads); long runs of
+// rows lose to the few spills that budget causes (4.6 -> 5.6 ms) and keep
+// the compiler's own choice (232 registers, two waves).
+template <typename T, int NMAX, int MINB>
+__global__ __launch_bounds__(64 * DSCAN_MAX_WAVES, MINB)
+void delta_scan_kernel(
     float* __restrict__ out, const T* __restrict__ q, int64_t q_s0,
     int64_t q_s1, const T* __restrict__ k, int64_t k_s0, int64_t k_s1,
     const T* __restrict__ v, int64_t v_s0, int64_t v_s1,
@@ -171,9 +178,11 @@ void delta_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
   const int waves = std::min(tiles, DSCAN_MAX_WAVES);
   const dim3 grid((tiles + waves - 1) / waves, H, S);
   const dim3 block(64 * waves);
-#define LAUNCH_DSCAN(NM)                                                      \
+  // mostly single rows: the three-wave build
+  const bool lean = T <= 2 * S;
+#define LAUNCH_DSCAN_B(NM, MB)                                                \
   hipLaunchKernelGGL(                                                         \
-      (delta_scan_kernel<act_t, NM>), grid, block, 0, stream,                 \
+      (delta_scan_kernel<act_t, NM, MB>), grid, block, 0, stream,             \
       (float*)out.data_ptr(), (const act_t*)q.data_ptr(),                     \
       (int64_t)q.stride(0), (int64_t)q.stride(1),                             \
       (const act_t*)k.data_ptr(), (int64_t)k.stride(0),                       \
@@ -184,14 +193,20 @@ void delta_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
       (const int32_t*)seq_start.data_ptr(),                                   \
       (const int32_t*)seq_slots.data_ptr(), H, G, N, P, (float)unit_eps,      \
       (float)qscale)
+#define LAUNCH_DSCAN(NM)                                                      \
+  do {                                                                        \
+    if (lean) LAUNCH_DSCAN_B(NM, 3);                                          \
+    else LAUNCH_DSCAN_B(NM, 1);                                               \
+  } while (0)
   IGW_DISPATCH_ACT(v, {
     if (N <= 16) LAUNCH_DSCAN(16);
     else if (N <= 32) LAUNCH_DSCAN(32);
     else if (N <= 64) LAUNCH_DSCAN(64);
     else if (N <= 128) LAUNCH_DSCAN(128);
-    else LAUNCH_DSCAN(256);
+    else LAUNCH_DSCAN_B(256, 1);
   });
 #undef LAUNCH_DSCAN
+#undef LAUNCH_DSCAN_B
   HIP_CHECK_KERNEL();
 }
 

@@ -983,3 +983,24 @@ def test_trace_command(tmp_path):
     assert not (tmp_path / "o" / "1.f32").exists()
     close(g0, ra[[0, 4]], 2e-4)
     close(g2, np.stack([ra[8], rb[3]]), 2e-4)
+
+
+def test_bench_configurations_are_comparable():
+    """The speed comparison runs both models at equal width, head sizes
+    and active feed-forward size."""
+    root = Path(__file__).resolve().parent.parent
+    sys.path.insert(0, str(root / "tools"))
+    try:
+        import bench_bozolorn as bb
+    finally:
+        sys.path.pop(0)
+    for sz in bb.SIZES.values():
+        boz, fdi = bb._configs(sz)
+        assert boz.hidden_size == fdi.hidden_size == sz["width"]
+        assert boz.num_layers == fdi.num_layers
+        moe = boz.layers[0].mlp
+        assert moe.expert_ff * moe.top == fdi.layers[0].mlp.ff
+        a, f = boz.layers[0].mixer.left, fdi.layers[0].mixer.left
+        assert (a.heads, a.kv_heads, a.dim, a.vdim) == (
+            f.heads, f.kv_heads, f.dim, f.vdim)
+        assert boz.layers[3].mixer.kv_from == 1
